@@ -6,6 +6,7 @@ from .blip2 import Blip2Config, Blip2ForConditionalGeneration
 from .registry import load_pretrained, model_class_for, register_model, registered_models
 from .kipirax import KipiraxConfig, KipiraxForCausalLM
 from .mubutar import MubutarConfig, MubutarForCausalLM
+from .vitinex import VitinexConfig, VitinexForCausalLM
 from .llama import LLAMA_CONFIGS, LlamaConfig, LlamaForCausalLM, llama_flops_per_token
 from .bert import BERT_CONFIGS, BertConfig, BertForMaskedLM, BertForSequenceClassification
 from .opt import OPT_CONFIGS, OPTConfig, OPTForCausalLM
@@ -19,7 +20,7 @@ from .vit import VIT_CONFIGS, ViTConfig, ViTForImageClassification
 from .whisper import WHISPER_CONFIGS, WhisperConfig, WhisperForConditionalGeneration
 
 __all__ = ["load_pretrained", "model_class_for", "register_model", "registered_models",
-           "KipiraxConfig", "KipiraxForCausalLM", "MubutarConfig", "MubutarForCausalLM",
+           "KipiraxConfig", "KipiraxForCausalLM", "MubutarConfig", "MubutarForCausalLM", "VitinexConfig", "VitinexForCausalLM",
            "LlamaConfig", "LlamaForCausalLM", "LLAMA_CONFIGS", "llama_flops_per_token",
            "OPTConfig", "OPTForCausalLM", "OPT_CONFIGS",
            "BertConfig", "BertForMaskedLM", "BertForSequenceClassification", "BERT_CONFIGS",

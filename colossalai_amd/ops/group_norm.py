@@ -8,7 +8,14 @@ norm. ``head_rms_norm_gate`` normalises every head vector of a ``[N, H, D]``
 tensor with one shared ``[D]`` weight and optionally multiplies by
 ``sigmoid(gate)``. ``add_rms_norm`` serves pre-norm layers: it adds one or two
 sublayer outputs to the float32 residual stream in place and hands back the
-RMS-normed stream for the next layer in one pass. All statistics are float32.
+RMS-normed stream for the next layer in one pass. ``gated_grouped_rms_norm``
+multiplies a row by ``silu(gate)`` *before* its grouped RMS norm (the output norm
+of a state-space mixer). ``layer_norm`` is the centred norm with a weight and no
+bias, ``(x - mean) / sqrt(var + eps) * w``; ``add_layer_norm`` serves layers that
+norm a sublayer's output on its way into the residual stream and norm the
+stream again for the next sublayer: ``residual += mult * layer_norm(y) * w_out``
+in place and, when ``w_next`` is given, ``layer_norm(residual) * w_next`` in one
+launch. All statistics are float32.
 """
 
 from typing import Optional
@@ -18,7 +25,9 @@ import torch
 from ._kernels import serving_kernels, use_serving_hip as use_hip
 
 __all__ = ["grouped_rms_norm", "grouped_rms_norm_ref", "head_rms_norm_gate", "head_rms_norm_gate_ref",
-           "merge_rms_norm", "merge_rms_norm_ref", "add_rms_norm", "add_rms_norm_ref"]
+           "merge_rms_norm", "merge_rms_norm_ref", "add_rms_norm", "add_rms_norm_ref",
+           "gated_grouped_rms_norm", "gated_grouped_rms_norm_ref", "layer_norm", "layer_norm_ref",
+           "add_layer_norm", "add_layer_norm_ref"]
 
 
 def grouped_rms_norm_ref(x, weight, groups: int, eps: float, residual=None, out_dtype=None):
@@ -35,8 +44,9 @@ def grouped_rms_norm(x, weight, groups: int, eps: float, residual: Optional[torc
     assert x.shape[-1] % groups == 0, "feature axis must split evenly into the norm groups"
     if use_hip(x):
         assert residual is None or residual.dtype == torch.float32
-        return serving_kernels().grouped_rms_norm(x.contiguous(), weight, groups, eps, residual,
-                                                  out_dtype or x.dtype)
+        if residual is not None or x.stride(-1) != 1:
+            x = x.contiguous()  # without a residual the kernel takes strided rows
+        return serving_kernels().grouped_rms_norm(x, weight, groups, eps, residual, out_dtype or x.dtype)
     return grouped_rms_norm_ref(x, weight, groups, eps, residual, out_dtype)
 
 
@@ -90,3 +100,50 @@ def add_rms_norm(residual, a, b, weight, eps: float, out_dtype=None):
         return serving_kernels().add_rms_norm(residual, a.contiguous(), None if b is None else b.contiguous(),
                                               weight, eps, out_dtype or a.dtype)
     return add_rms_norm_ref(residual, a, b, weight, eps, out_dtype)
+
+
+def gated_grouped_rms_norm_ref(x, gate, weight, groups: int, eps: float, out_dtype=None):
+    g = gate.float()
+    return grouped_rms_norm_ref(x.float() * (g * torch.sigmoid(g)), weight, groups, eps, None, out_dtype or gate.dtype)
+
+
+def gated_grouped_rms_norm(x, gate, weight, groups: int, eps: float, out_dtype=None):
+    """x [N, W] (float32 or an activation type), gate [N, W] logits (rows may be strided): the row
+    ``x * silu(gate)`` is RMS-normed in ``groups`` equal parts and weighted. The gate comes before the norm."""
+    assert x.shape[-1] % groups == 0 and gate.shape == x.shape
+    if use_hip(x):
+        return serving_kernels().gated_grouped_rms_norm(x, gate, weight, groups, eps, out_dtype or gate.dtype)
+    return gated_grouped_rms_norm_ref(x, gate, weight, groups, eps, out_dtype)
+
+
+def layer_norm_ref(x, weight, eps: float, out_dtype=None):
+    xf = x.float()
+    mu = xf.mean(-1, keepdim=True)
+    d = xf - mu
+    return (d * torch.rsqrt(d.pow(2).mean(-1, keepdim=True) + eps) * weight.float()).to(out_dtype or x.dtype)
+
+
+def layer_norm(x, weight, eps: float, out_dtype=None):
+    """Centred norm of the rows of x [N, W] with a weight and no bias; the variance is the mean of the squared
+    deviations (two passes over the row, float32)."""
+    if use_hip(x):
+        return serving_kernels().add_layer_norm(None, x.contiguous(), None, 1.0, weight, eps, out_dtype or x.dtype)
+    return layer_norm_ref(x, weight, eps, out_dtype)
+
+
+def add_layer_norm_ref(residual, y, w_out, mult: float, w_next, eps: float, out_dtype=None):
+    residual.add_(layer_norm_ref(y, w_out, eps, torch.float32), alpha=mult)
+    if w_next is None:
+        return None
+    return layer_norm_ref(residual, w_next, eps, out_dtype or y.dtype)
+
+
+def add_layer_norm(residual, y, w_out, mult: float, w_next, eps: float, out_dtype=None):
+    """``residual += mult * layer_norm(y) * w_out`` in place (float32 [N, W]; ``y`` a sublayer's output of any
+    activation type), then, when ``w_next`` is given, returns ``layer_norm(residual) * w_next`` in ``out_dtype``:
+    the input of the next sublayer. With ``w_next=None`` only the sum is formed."""
+    if use_hip(residual):
+        assert residual.dtype == torch.float32
+        return serving_kernels().add_layer_norm(residual, y.contiguous(), w_out, float(mult), w_next, eps,
+                                                out_dtype or y.dtype)
+    return add_layer_norm_ref(residual, y, w_out, mult, w_next, eps, out_dtype)

@@ -2,7 +2,7 @@
 
 Every head keeps a float32 matrix ``S [D, Dv]`` per state slot (rows = key /
 query channels, columns = value channels) that is carried from step to step.
-Two update rules are provided:
+Three update rules are provided:
 
 * ``gated_delta_rule`` — per-channel decay plus delta-rule write
   ``S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q``
@@ -12,6 +12,11 @@ Two update rules are provided:
 * ``tied_gate_recurrence`` (HGRN2) — the forget gate also sets the write:
   ``S <- diag(f) S + (1 - f) v^T;  o = S^T q`` with
   ``f = lower + (1 - lower) sigmoid(f_logit + f_bias)`` and ``q = silu(.)``.
+
+* ``ssd_recurrence`` (state-space duality) — one decay per head and token:
+  ``S <- a S + dt B x^T;  y = S^T C + D_skip x`` with ``dt = softplus(dt_raw +
+  dt_bias)``, ``a = exp(-exp(A_log_h) dt)``; ``B`` and ``C`` are shared by the
+  heads of a group (head ``h`` reads group ``h // (H / G)``).
 
 The read-out always includes the current token's write. Gates, decays and the
 state are float32 whatever the activation dtype is.
@@ -23,7 +28,8 @@ import torch.nn.functional as F
 from ._kernels import serving_state_kernels as serving_kernels, use_serving_hip as use_hip
 from .ragged import RaggedBatch
 
-__all__ = ["gated_delta_rule", "gated_delta_rule_ref", "tied_gate_recurrence", "tied_gate_recurrence_ref"]
+__all__ = ["gated_delta_rule", "gated_delta_rule_ref", "tied_gate_recurrence", "tied_gate_recurrence_ref",
+           "ssd_recurrence", "ssd_recurrence_ref"]
 
 
 def _scan_ref(batch, state, n_out, step):
@@ -98,3 +104,33 @@ def tied_gate_recurrence(q, f_logit, v, f_bias, lower, state, batch: RaggedBatch
         return serving_kernels().tied_gate_recurrence(q, f_logit, v, f_bias, lower, state, batch.cu, batch.start,
                                                       batch.slots)
     return tied_gate_recurrence_ref(q, f_logit, v, f_bias, lower, state, batch)
+
+
+def ssd_recurrence_ref(x, B, C, dt_raw, A_log, dt_bias, D_skip, state, batch: RaggedBatch):
+    N, H, Dv = x.shape
+    G = B.shape[1]
+    rep = H // G
+    xf = x.float()
+    Bf = B.float().repeat_interleave(rep, 1)   # [N, H, D]
+    Cf = C.float().repeat_interleave(rep, 1)
+    dt = F.softplus(dt_raw.float() + dt_bias.float(), threshold=1e30)    # [N, H], no clamp of large arguments
+    a = torch.exp(-torch.exp(A_log.float())[None, :] * dt)
+    skip = D_skip.float()[:, None]
+    out = torch.empty(N, H, Dv, dtype=torch.float32, device=x.device)
+
+    def step(S, t):
+        S = a[t][:, None, None] * S + (dt[t][:, None] * Bf[t])[:, :, None] * xf[t][:, None, :]
+        out[t] = torch.einsum("hdv,hd->hv", S, Cf[t]) + skip * xf[t]
+        return S
+
+    _scan_ref(batch, state, out, step)
+    return out
+
+
+def ssd_recurrence(x, B, C, dt_raw, A_log, dt_bias, D_skip, state, batch: RaggedBatch):
+    """x [N, H, Dv]; B, C [N, G, D] (H a multiple of G; rows may be strided); dt_raw [N, H]; A_log, dt_bias,
+    D_skip [H]; state [slots, H, D, Dv] float32. Returns y [N, H, Dv] float32."""
+    if use_hip(x):
+        return serving_kernels().ssd_recurrence(x, B, C, dt_raw, A_log, dt_bias, D_skip, state, batch.cu,
+                                                batch.start, batch.slots)
+    return ssd_recurrence_ref(x, B, C, dt_raw, A_log, dt_bias, D_skip, state, batch)

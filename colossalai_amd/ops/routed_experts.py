@@ -13,6 +13,10 @@ weights:
 * the ``top`` largest remaining choice scores are chosen (ties go to the lower
   index) and their plain scores are divided by their sum plus ``renorm_eps``.
 
+With ``score="softmax"`` the scores are the softmax of the logits over all
+experts, and with ``renorm=False`` the chosen scores are the mixing weights as
+they are.
+
 ``routed_expert_ffn`` runs ``down_e(act(up_e(h)))`` for each token's chosen
 experts and forms ``base + sum_j weight_j * y_j`` in float32. On the GPU nothing
 of a bfloat16 step goes to the host: a small step (decode tokens) streams just
@@ -44,10 +48,10 @@ GEMV_FALLBACK_PAIRS = 2048
 
 
 def grouped_topk_route_ref(logits, correction, top: int, group_count: int = 1, group_keep: int = 1,
-                           group_top: int = 2, renorm_eps: float = 1e-20):
+                           group_top: int = 2, renorm_eps: float = 1e-20, score: str = "sigmoid", renorm: bool = True):
     N, E = logits.shape
-    s = torch.sigmoid(logits.float())
-    choice = s + correction.float()
+    s = torch.softmax(logits.float(), -1) if score == "softmax" else torch.sigmoid(logits.float())
+    choice = s + correction.float() if correction is not None else s
     if group_count > 1:
         per = E // group_count
         grouped = choice.view(N, group_count, per)
@@ -59,19 +63,26 @@ def grouped_topk_route_ref(logits, correction, top: int, group_count: int = 1, g
         choice = grouped.masked_fill(~allowed[:, :, None], float("-inf")).reshape(N, E)
     idx = torch.sort(choice, dim=-1, descending=True, stable=True).indices[:, :top]
     w = s.gather(1, idx)
-    return idx.int(), w / (w.sum(-1, keepdim=True) + renorm_eps)
+    return idx.int(), (w / (w.sum(-1, keepdim=True) + renorm_eps) if renorm else w)
+
+
+SCORES = {"sigmoid": 0, "softmax": 1}
 
 
 def grouped_topk_route(logits, correction, top: int, group_count: int = 1, group_keep: int = 1,
-                       group_top: int = 2, renorm_eps: float = 1e-20):
-    """logits [N, E] float32, correction [E] -> (ids [N, top] int32, weights [N, top] float32)."""
+                       group_top: int = 2, renorm_eps: float = 1e-20, score: str = "sigmoid", renorm: bool = True):
+    """logits [N, E] float32 (rows may be strided), correction [E] or None -> (ids [N, top] int32, weights
+    [N, top] float32). ``score``: "sigmoid" or "softmax" (over all experts); ``renorm``: divide the chosen scores
+    by their sum."""
     N, E = logits.shape
+    assert score in SCORES
     assert E % group_count == 0 and 0 < group_keep <= group_count
     assert 0 < top <= (E // group_count) * group_keep, "fewer experts in the kept groups than are to be chosen"
     if use_hip(logits):
-        return serving_kernels().grouped_topk_route(logits.float().contiguous(), correction, top, group_count,
-                                                    group_keep, group_top, renorm_eps)
-    return grouped_topk_route_ref(logits, correction, top, group_count, group_keep, group_top, renorm_eps)
+        return serving_kernels().grouped_topk_route(logits.float(), correction, top, group_count,
+                                                    group_keep, group_top, renorm_eps, SCORES[score], renorm)
+    return grouped_topk_route_ref(logits, correction, top, group_count, group_keep, group_top, renorm_eps, score,
+                                  renorm)
 
 
 def _act(x, activation: str):
@@ -80,9 +91,12 @@ def _act(x, activation: str):
     raise ValueError(f"unknown expert activation {activation!r}")
 
 
-def routed_expert_ffn_ref(h, w_up, w_down, ids, weights, base=None, activation: str = "relu_squared"):
+def routed_expert_ffn_ref(h, w_up, w_down, ids, weights, base=None, activation: str = "relu_squared",
+                          base_gate=None):
     N, top = ids.shape
     out = torch.zeros(N, w_down.shape[1], dtype=torch.float32, device=h.device) if base is None else base.float().clone()
+    if base is not None and base_gate is not None:
+        out = out * torch.sigmoid(base_gate.float().reshape(N, 1))
     for e in range(w_up.shape[0]):
         rows, slot = (ids == e).nonzero(as_tuple=True)
         if rows.numel():
@@ -107,7 +121,7 @@ def _sort_pairs(ids, E: int):
 SORT_KERNEL_MAX_PAIRS = 8192  # the one-block sort kernel holds a step's ids in LDS
 
 
-def _grouped_expert_ffn(h, w_up, w_down, ids, weights, base):
+def _grouped_expert_ffn(h, w_up, w_down, ids, weights, base, base_gate=None):
     """One grouped matrix-core launch per product; the up product gathers the tokens' rows itself and squares the
     rectified accumulator. Steps of up to 8192 pairs are sorted by one kernel, larger ones by library sorts."""
     N, top = ids.shape
@@ -119,10 +133,10 @@ def _grouped_expert_ffn(h, w_up, w_down, ids, weights, base):
         src, inv = (order // top).int(), inv.int().view(N, top)
     hidden = K.expert_grouped_gemm(h, src, w_up, offsets, ids.numel(), True)
     y = K.expert_grouped_gemm(hidden, None, w_down, offsets, ids.numel(), False)
-    return K.expert_combine(y, inv, weights, base)
+    return K.expert_combine(y, inv, weights, base, base_gate)
 
 
-def _sorted_expert_ffn(h, w_up, w_down, ids, weights, base, activation):
+def _sorted_expert_ffn(h, w_up, w_down, ids, weights, base, activation, base_gate=None):
     """Pairs sorted by expert, one up and one down library product per expert that got rows (their row counts come
     to the host), then every token gathers its ``top`` results in slot order."""
     N, top = ids.shape
@@ -140,7 +154,7 @@ def _sorted_expert_ffn(h, w_up, w_down, ids, weights, base, activation):
         lo, hi = bounds[e], bounds[e + 1]
         if hi > lo:
             torch.mm(hidden[lo:hi], w_down[e].t(), out=y[lo:hi])
-    return serving_kernels().expert_combine(y, inv.int().view(N, top), weights, base)
+    return serving_kernels().expert_combine(y, inv.int().view(N, top), weights, base, base_gate)
 
 
 def _grouped_fits(h, w_up, w_down) -> bool:
@@ -149,19 +163,21 @@ def _grouped_fits(h, w_up, w_down) -> bool:
 
 
 def routed_expert_ffn(h, w_up, w_down, ids, weights, base: Optional[torch.Tensor] = None,
-                      activation: str = "relu_squared"):
+                      activation: str = "relu_squared", base_gate: Optional[torch.Tensor] = None):
     """h [N, W]; w_up [E, F, W]; w_down [E, W, F]; ids [N, top] int32; weights
     [N, top] float32; ``base`` [N, W] (any activation type) is added, e.g. a
-    shared expert's output. Returns float32 [N, W]."""
+    shared expert's output, multiplied by ``sigmoid(base_gate)`` when
+    ``base_gate`` ([N] float32 logits, any stride) is given. Returns float32 [N, W]."""
     if not use_hip(h):
-        return routed_expert_ffn_ref(h, w_up, w_down, ids, weights, base, activation)
+        return routed_expert_ffn_ref(h, w_up, w_down, ids, weights, base, activation, base_gate)
+    assert base_gate is None or (base is not None and base_gate.dtype == torch.float32 and base_gate.numel() == h.shape[0])
     if activation != "relu_squared":
         raise ValueError(f"unknown expert activation {activation!r}")
     h = h.contiguous()
     if ids.numel() <= GEMV_MAX_PAIRS:
-        return serving_kernels().expert_ffn_gemv(h, w_up, w_down, ids, weights, base)
+        return serving_kernels().expert_ffn_gemv(h, w_up, w_down, ids, weights, base, base_gate)
     if _grouped_fits(h, w_up, w_down):
-        return _grouped_expert_ffn(h, w_up, w_down, ids, weights, base)
+        return _grouped_expert_ffn(h, w_up, w_down, ids, weights, base, base_gate)
     if ids.numel() <= GEMV_FALLBACK_PAIRS:
-        return serving_kernels().expert_ffn_gemv(h, w_up, w_down, ids, weights, base)
-    return _sorted_expert_ffn(h, w_up, w_down, ids, weights, base, activation)
+        return serving_kernels().expert_ffn_gemv(h, w_up, w_down, ids, weights, base, base_gate)
+    return _sorted_expert_ffn(h, w_up, w_down, ids, weights, base, activation, base_gate)
