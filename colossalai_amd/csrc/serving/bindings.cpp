@@ -24,11 +24,22 @@ at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at:
 at::Tensor silu_mul(at::Tensor packed);
 c10::optional<at::Tensor> add_rms_norm(at::Tensor residual, at::Tensor a, c10::optional<at::Tensor> b,
                                        c10::optional<at::Tensor> weight, double eps, at::ScalarType out_dtype);
-std::vector<at::Tensor> grouped_topk_route(at::Tensor logits, at::Tensor correction, int64_t top, int64_t group_count,
-                                           int64_t group_keep, int64_t group_top, double renorm_eps);
+std::vector<at::Tensor> grouped_topk_route(at::Tensor logits, c10::optional<at::Tensor> correction, int64_t top,
+                                           int64_t group_count, int64_t group_keep, int64_t group_top,
+                                           double renorm_eps, int64_t score_fn, bool renorm);
 at::Tensor expert_ffn_gemv(at::Tensor h, at::Tensor w_up, at::Tensor w_down, at::Tensor ids, at::Tensor weights,
-                           c10::optional<at::Tensor> base);
-at::Tensor expert_combine(at::Tensor y, at::Tensor inv, at::Tensor weights, c10::optional<at::Tensor> base);
+                           c10::optional<at::Tensor> base, c10::optional<at::Tensor> base_gate);
+at::Tensor expert_combine(at::Tensor y, at::Tensor inv, at::Tensor weights, c10::optional<at::Tensor> base,
+                          c10::optional<at::Tensor> base_gate);
+at::Tensor gelu_tanh_mul(at::Tensor packed);
+at::Tensor gated_grouped_rms_norm(at::Tensor x, at::Tensor gate, at::Tensor weight, int64_t groups, double eps,
+                                  at::ScalarType out_dtype);
+c10::optional<at::Tensor> add_layer_norm(c10::optional<at::Tensor> residual, at::Tensor y,
+                                         c10::optional<at::Tensor> w_out, double mult,
+                                         c10::optional<at::Tensor> w_next, double eps, at::ScalarType out_dtype);
+void rotate_pairs(at::Tensor x, at::Tensor positions, at::Tensor freqs, at::Tensor out);
+void latent_kv_write(at::Tensor dkv, at::Tensor norm_w, double eps, at::Tensor freqs, at::Tensor positions,
+                     at::Tensor pool, at::Tensor rows);
 std::vector<at::Tensor> expert_sort(at::Tensor ids, int64_t num_experts);
 at::Tensor expert_grouped_gemm(at::Tensor a, c10::optional<at::Tensor> a_rows, at::Tensor w, at::Tensor offsets,
                                int64_t rows, bool relu_squared);
@@ -48,7 +59,14 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("paged_attention", &s::paged_attention, "ragged paged attention: window, kept prefix, distance bias, gate, soft cap, sink");
   m.def("silu_mul", &s::silu_mul, "silu(gate) * up of a packed [N, 2F] tensor");
   m.def("add_rms_norm", &s::add_rms_norm, "residual += a (+ b) in place, then the RMS norm of the sum");
-  m.def("grouped_topk_route", &s::grouped_topk_route, "sigmoid router: correction, group-limited top-k, renormalised");
+  m.def("grouped_topk_route", &s::grouped_topk_route,
+        "sigmoid or softmax router: correction, group-limited top-k, renormalised or not");
+  m.def("gelu_tanh_mul", &s::gelu_tanh_mul, "gelu_tanh(gate) * up of a packed [N, 2F] tensor");
+  m.def("gated_grouped_rms_norm", &s::gated_grouped_rms_norm, "x * silu(gate), then grouped RMS norm");
+  m.def("add_layer_norm", &s::add_layer_norm,
+        "residual += mult * layer_norm(y) * w_out in place, then the layer norm of the sum (weight, no bias)");
+  m.def("rotate_pairs", &s::rotate_pairs, "rotary positions on neighbouring pairs, strided in and out");
+  m.def("latent_kv_write", &s::latent_kv_write, "latent row: RMS norm + pair rotation + scatter into pool rows");
   m.def("expert_ffn_gemv", &s::expert_ffn_gemv, "chosen experts' feed-forward of a small step, matrix-vector kernels");
   m.def("expert_sort", &s::expert_sort, "stable sort of (token, expert) pairs by expert: offsets, source tokens, inverse");
   m.def("expert_grouped_gemm", &s::expert_grouped_gemm,

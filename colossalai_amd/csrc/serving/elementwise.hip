@@ -1,6 +1,7 @@
 // Element-wise serving kernels: token shift with carried previous row,
-// squared ReLU, gated SiLU of a packed tensor, logit soft-cap, ragged scatter
-// of keys/values into pages.
+// squared ReLU, gated SiLU / tanh-GELU of a packed tensor, logit soft-cap, ragged
+// scatter of keys/values into pages, rotary positions on neighbouring pairs, and
+// the write of a latent-attention row (norm + rotation + scatter).
 #include "serving_common.h"
 
 namespace cai {
@@ -137,7 +138,14 @@ void paged_kv_write(at::Tensor k, at::Tensor v, at::Tensor kpool, at::Tensor vpo
 
 // packed [N, 2F] = [gate | up], rows strided by ps -> out [N, F] = silu(gate) * up, formed in float32.
 // VEC: eight elements per thread (F and the row stride are multiples of 8 and the base is aligned).
-template <typename T, bool VEC>
+// ACT: 0 = silu(g) = g * sigmoid(g); 1 = the tanh form of GELU, 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))).
+template <int ACT>
+DEV_INLINE float gate_act(float g) {
+  if (ACT == 0) return g * sigmoidf_(g);
+  return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+}
+
+template <typename T, bool VEC, int ACT>
 __global__ __launch_bounds__(256) void silu_mul_kernel(T* __restrict__ out, const T* __restrict__ packed, long ps,
                                                        long N, int F) {
   constexpr int PER = VEC ? 8 : 1;
@@ -150,16 +158,17 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(T* __restrict__ out, cons
       load8(packed + n * ps + f, g);
       load8(packed + n * ps + F + f, u);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) g[e] = g[e] * sigmoidf_(g[e]) * u[e];
+      for (int e = 0; e < 8; ++e) g[e] = gate_act<ACT>(g[e]) * u[e];
       store8(out + n * F + f, g);
     } else {
       const float g = ldf(packed + n * ps + f), u = ldf(packed + n * ps + F + f);
-      stf(out + i, g * sigmoidf_(g) * u);
+      stf(out + i, gate_act<ACT>(g) * u);
     }
   }
 }
 
-at::Tensor silu_mul(at::Tensor packed) {
+template <int ACT>
+static at::Tensor gated_act_mul(at::Tensor packed) {
   check_act(packed, "packed");
   TORCH_CHECK(packed.dim() == 2 && packed.stride(1) == 1 && packed.size(1) % 2 == 0, "packed must be [N, 2F] with dense rows");
   const long N = packed.size(0);
@@ -169,14 +178,141 @@ at::Tensor silu_mul(at::Tensor packed) {
   const bool vec = F % 8 == 0 && packed.stride(0) % 8 == 0 && reinterpret_cast<uintptr_t>(packed.data_ptr()) % 32 == 0;
   SERVING_DISPATCH_ACT(packed, T, {
     if (vec)
-      hipLaunchKernelGGL((silu_mul_kernel<T, true>), dim3(capped_grid((N * F / 8 + 255) / 256, 8192)), dim3(256), 0, stream(),
+      hipLaunchKernelGGL((silu_mul_kernel<T, true, ACT>), dim3(capped_grid((N * F / 8 + 255) / 256, 8192)), dim3(256), 0, stream(),
                          ptr<T>(out), ptr<T>(packed), (long)packed.stride(0), N, F);
     else
-      hipLaunchKernelGGL((silu_mul_kernel<T, false>), dim3(capped_grid((N * F + 255) / 256, 4096)), dim3(256), 0, stream(),
+      hipLaunchKernelGGL((silu_mul_kernel<T, false, ACT>), dim3(capped_grid((N * F + 255) / 256, 4096)), dim3(256), 0, stream(),
                          ptr<T>(out), ptr<T>(packed), (long)packed.stride(0), N, F);
   });
   HIP_CHECK_LAST();
   return out;
+}
+
+at::Tensor silu_mul(at::Tensor packed) { return gated_act_mul<0>(packed); }
+at::Tensor gelu_tanh_mul(at::Tensor packed) { return gated_act_mul<1>(packed); }
+
+// ------------------------------------------------------------ rotary on pairs
+// The pair (2i, 2i + 1), i < half, of a vector at position p turns by a = p * freqs[i], float32.
+DEV_INLINE void turn_pair(float u, float v, float a, float& ou, float& ov) {
+  float sn, cs;
+  sincosf(a, &sn, &cs);
+  ou = u * cs - v * sn;
+  ov = v * cs + u * sn;
+}
+
+// x element (n, h, r) at n*xs + h*xh + r; out likewise with its own strides. One thread per pair
+// (or single trailing channel when R is odd); channels from 2 * half on are copied.
+template <typename T>
+__global__ __launch_bounds__(256) void rotate_pairs_kernel(
+    T* __restrict__ out, long os, long oh, const T* __restrict__ x, long xs, long xh, const int* __restrict__ positions,
+    const float* __restrict__ freqs, long N, int H, int R, int half) {
+  const int per = (R + 1) / 2;
+  const long total = N * H * per;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    const int j = (int)(i % per);
+    const long nh = i / per;
+    const int h = (int)(nh % H);
+    const long n = nh / H;
+    const T* src = x + n * xs + h * xh + 2 * j;
+    T* dst = out + n * os + h * oh + 2 * j;
+    const float u = ldf(src);
+    if (2 * j + 1 >= R) {
+      stf(dst, u);
+      continue;
+    }
+    const float v = ldf(src + 1);
+    if (j < half) {
+      float ou, ov;
+      turn_pair(u, v, (float)positions[n] * freqs[j], ou, ov);
+      stf(dst, ou);
+      stf(dst + 1, ov);
+    } else {
+      stf(dst, u);
+      stf(dst + 1, v);
+    }
+  }
+}
+
+void rotate_pairs(at::Tensor x, at::Tensor positions, at::Tensor freqs, at::Tensor out) {
+  check_act(x, "x"); check_act(out, "out");
+  TORCH_CHECK(x.dim() == 3 && out.dim() == 3 && x.sizes() == out.sizes() && x.scalar_type() == out.scalar_type());
+  TORCH_CHECK(x.stride(2) == 1 && out.stride(2) == 1, "channels must have unit stride");
+  check_i32(positions, "positions");
+  const long N = x.size(0);
+  const int H = (int)x.size(1), R = (int)x.size(2);
+  TORCH_CHECK(positions.numel() == N);
+  TORCH_CHECK(freqs.is_cuda() && is_f32(freqs) && freqs.is_contiguous() && 2 * freqs.numel() <= R,
+              "freqs must be float32 [dims / 2] with dims <= R");
+  if (N * H * R == 0) return;
+  const long total = N * H * ((R + 1) / 2);
+  SERVING_DISPATCH_ACT(x, T, {
+    hipLaunchKernelGGL(rotate_pairs_kernel<T>, dim3(capped_grid((total + 255) / 256, 8192)), dim3(256), 0, stream(),
+                       ptr<T>(out), (long)out.stride(0), (long)out.stride(1), ptr<T>(x), (long)x.stride(0),
+                       (long)x.stride(1), positions.data_ptr<int>(), freqs.data_ptr<float>(), N, H, R,
+                       (int)freqs.numel());
+  });
+  HIP_CHECK_LAST();
+}
+
+// ------------------------------------------------------------- latent row write
+// One wave per token: dkv row [rank + R] (row-strided) -> pool row rows[n]: the first `rank`
+// channels RMS-normed with a weight (float32 statistics), the last R rotated pair-wise (the
+// first 2 * half of them) by the token's position.
+template <typename T>
+__global__ __launch_bounds__(256) void latent_kv_write_kernel(
+    T* __restrict__ pool, const T* __restrict__ dkv, long ds, const float* __restrict__ w,
+    const float* __restrict__ freqs, const int* __restrict__ positions, const int* __restrict__ rows, long N, int rank,
+    int R, int half, float eps) {
+  const int lane = threadIdx.x & 63;
+  const long n = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (n >= N) return;
+  const T* src = dkv + n * ds;
+  T* dst = pool + (long)rows[n] * (rank + R);
+  float ssq = 0.0f;
+#pragma unroll 4
+  for (int i = lane; i < rank; i += 64) {
+    const float v = ldf(src + i);
+    ssq += v * v;
+  }
+  ssq = wave_reduce_sum(ssq);
+  const float inv = 1.0f / sqrtf(ssq / (float)rank + eps);
+#pragma unroll 4
+  for (int i = lane; i < rank; i += 64) stf(dst + i, ldf(src + i) * inv * w[i]);
+  const float p = (float)positions[n];
+  for (int j = lane; 2 * j < R; j += 64) {
+    const float u = ldf(src + rank + 2 * j);
+    if (2 * j + 1 >= R) {
+      stf(dst + rank + 2 * j, u);
+      continue;
+    }
+    float v = ldf(src + rank + 2 * j + 1), ou = u, ov = v;
+    if (j < half) turn_pair(u, v, p * freqs[j], ou, ov);
+    stf(dst + rank + 2 * j, ou);
+    stf(dst + rank + 2 * j + 1, ov);
+  }
+}
+
+void latent_kv_write(at::Tensor dkv, at::Tensor norm_w, double eps, at::Tensor freqs, at::Tensor positions,
+                     at::Tensor pool, at::Tensor rows) {
+  check_act(dkv, "dkv");
+  TORCH_CHECK(dkv.dim() == 2 && dkv.stride(1) == 1, "dkv must be [N, rank + R] with unit inner stride");
+  TORCH_CHECK(pool.is_cuda() && pool.is_contiguous() && pool.dim() == 4 && pool.size(2) == 1 &&
+              pool.size(3) == dkv.size(1) && pool.scalar_type() == dkv.scalar_type(),
+              "pool must be contiguous [pages, page, 1, rank + R] of dkv's dtype");
+  check_i32(positions, "positions"); check_i32(rows, "rows");
+  const long N = dkv.size(0);
+  at::Tensor w = f32c(norm_w);
+  const int rank = (int)w.numel(), R = (int)dkv.size(1) - rank;
+  TORCH_CHECK(rank > 0 && R >= 0 && positions.numel() == N && rows.numel() == N);
+  TORCH_CHECK(freqs.is_cuda() && is_f32(freqs) && freqs.is_contiguous() && 2 * freqs.numel() <= R,
+              "freqs must be float32 [dims / 2] with dims <= R");
+  if (N == 0) return;
+  SERVING_DISPATCH_ACT(dkv, T, {
+    hipLaunchKernelGGL(latent_kv_write_kernel<T>, dim3((unsigned)((N + 3) / 4)), dim3(256), 0, stream(), ptr<T>(pool),
+                       ptr<T>(dkv), (long)dkv.stride(0), w.data_ptr<float>(), freqs.data_ptr<float>(),
+                       positions.data_ptr<int>(), rows.data_ptr<int>(), N, rank, R, (int)freqs.numel(), (float)eps);
+  });
+  HIP_CHECK_LAST();
 }
 
 }  // namespace serving

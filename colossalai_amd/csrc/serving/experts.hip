@@ -1,6 +1,6 @@
 // Mixture-of-experts serving kernels:
-//   grouped_topk_route : sigmoid scores, a selection-only correction, group-limited
-//                        top-k with ties to the lower index, chosen scores renormalised;
+//   grouped_topk_route : sigmoid (or softmax) scores, a selection-only correction, group-limited
+//                        top-k with ties to the lower index, chosen scores renormalised (or kept);
 //   expert_ffn_gemv    : a small step's chosen experts as two matrix-vector kernels
 //                        (up + squared ReLU per (token, expert) pair, then the weighted
 //                        down products of a token summed with its base row) — only the
@@ -19,8 +19,9 @@ namespace serving {
 // last token repeats the last token and writes nothing). LDS per wave: scores [E], choice
 // scores [E], group worths [groups], picked scores [top].
 __global__ __launch_bounds__(256) void grouped_topk_route_kernel(
-    int* __restrict__ ids, float* __restrict__ wts, const float* __restrict__ logits, const float* __restrict__ corr,
-    long N, int E, int top, int groups, int keep, int group_top, float eps) {
+    int* __restrict__ ids, float* __restrict__ wts, const float* __restrict__ logits, long ld,
+    const float* __restrict__ corr, long N, int E, int top, int groups, int keep, int group_top, float eps,
+    int softmax, int renorm) {
   extern __shared__ float lds[];
   const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
   float* sc = lds + (long)wid * (2 * E + groups + top);
@@ -30,10 +31,28 @@ __global__ __launch_bounds__(256) void grouped_topk_route_kernel(
   const long tok = (long)blockIdx.x * 4 + wid;
   const bool live = tok < N;
   const long n = live ? tok : N - 1;
-  for (int e = lane; e < E; e += 64) {
-    const float s = sigmoidf_(logits[n * E + e]);
-    sc[e] = s;
-    ch[e] = s + corr[e];
+  if (softmax) {  // over all experts, float32: exp(z - max) / sum
+    float mx = -INFINITY;
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, logits[n * ld + e]);
+    mx = wave_reduce_max(mx);
+    float sum = 0.0f;
+    for (int e = lane; e < E; e += 64) {
+      const float w = expf(logits[n * ld + e] - mx);
+      sc[e] = w;
+      sum += w;
+    }
+    sum = wave_reduce_sum(sum);
+    for (int e = lane; e < E; e += 64) {
+      const float s = sc[e] / sum;
+      sc[e] = s;
+      ch[e] = s + (corr != nullptr ? corr[e] : 0.0f);
+    }
+  } else {
+    for (int e = lane; e < E; e += 64) {
+      const float s = sigmoidf_(logits[n * ld + e]);
+      sc[e] = s;
+      ch[e] = s + (corr != nullptr ? corr[e] : 0.0f);
+    }
   }
   __syncthreads();
   if (groups > 1) {
@@ -91,27 +110,35 @@ __global__ __launch_bounds__(256) void grouped_topk_route_kernel(
     __syncthreads();
   }
   if (live)
-    for (int t = lane; t < top; t += 64) wts[tok * top + t] = pick[t] / (total + eps);
+    for (int t = lane; t < top; t += 64) wts[tok * top + t] = renorm ? pick[t] / (total + eps) : pick[t];
 }
 
-std::vector<at::Tensor> grouped_topk_route(at::Tensor logits, at::Tensor correction, int64_t top, int64_t group_count,
-                                           int64_t group_keep, int64_t group_top, double renorm_eps) {
-  TORCH_CHECK(logits.is_cuda() && is_f32(logits) && logits.dim() == 2 && logits.is_contiguous(),
-              "router logits must be contiguous float32 [N, E]");
+std::vector<at::Tensor> grouped_topk_route(at::Tensor logits, c10::optional<at::Tensor> correction, int64_t top,
+                                           int64_t group_count, int64_t group_keep, int64_t group_top,
+                                           double renorm_eps, int64_t score_fn, bool renorm) {
+  TORCH_CHECK(logits.is_cuda() && is_f32(logits) && logits.dim() == 2 && logits.stride(1) == 1,
+              "router logits must be float32 [N, E] with unit inner stride");
+  TORCH_CHECK(score_fn == 0 || score_fn == 1, "score function: 0 = sigmoid, 1 = softmax");
   const long N = logits.size(0);
   const int E = (int)logits.size(1);
   TORCH_CHECK(group_count >= 1 && E % group_count == 0 && group_keep >= 1 && group_keep <= group_count && group_top >= 1);
   TORCH_CHECK(top >= 1 && top <= (E / group_count) * group_keep, "more experts to choose than the kept groups hold");
-  at::Tensor corr = f32c(correction);
-  TORCH_CHECK(corr.numel() == E && corr.is_cuda());
+  at::Tensor corr;
+  const float* corrp = nullptr;
+  if (correction.has_value()) {
+    corr = f32c(*correction);
+    TORCH_CHECK(corr.numel() == E && corr.is_cuda());
+    corrp = corr.data_ptr<float>();
+  }
   at::Tensor ids = at::empty({N, top}, logits.options().dtype(at::kInt));
   at::Tensor wts = at::empty({N, top}, logits.options());
   if (N == 0) return {ids, wts};
   const size_t smem = (size_t)4 * (2 * E + group_count + top) * sizeof(float);
   TORCH_CHECK(smem <= 64 * 1024, "too many experts for the router kernel");
   hipLaunchKernelGGL(grouped_topk_route_kernel, dim3((unsigned)((N + 3) / 4)), dim3(256), smem, stream(),
-                     ids.data_ptr<int>(), wts.data_ptr<float>(), logits.data_ptr<float>(), corr.data_ptr<float>(), N, E,
-                     (int)top, (int)group_count, (int)group_keep, (int)group_top, (float)renorm_eps);
+                     ids.data_ptr<int>(), wts.data_ptr<float>(), logits.data_ptr<float>(), (long)logits.stride(0), corrp, N,
+                     E, (int)top, (int)group_count, (int)group_keep, (int)group_top, (float)renorm_eps, (int)score_fn,
+                     renorm ? 1 : 0);
   HIP_CHECK_LAST();
   return {ids, wts};
 }
@@ -172,15 +199,18 @@ __global__ __launch_bounds__(256) void expert_up_gemv_kernel(
   }
 }
 
-// block = (token, chunk of 4 * R output rows): out[n, w] = base[n, w] + sum_j weight_j down_{e_j}[w, :] . hidden[n, j, :]
+// block = (token, chunk of 4 * R output rows): out[n, w] = base[n, w] + sum_j weight_j down_{e_j}[w, :] . hidden[n, j, :];
+// with base_gate the base row is first multiplied by sigmoid(base_gate[n])
 template <typename T, typename TB>
 __global__ __launch_bounds__(256) void expert_down_gemv_kernel(
     float* __restrict__ out, const T* __restrict__ hidden, const T* __restrict__ w_down, const int* __restrict__ ids,
-    const float* __restrict__ weights, const TB* __restrict__ base, int top, int E, int F, int W, int vec) {
+    const float* __restrict__ weights, const TB* __restrict__ base, const float* __restrict__ base_gate, long bgs,
+    int top, int E, int F, int W, int vec) {
   const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const long n = blockIdx.x;
   const int row0 = (blockIdx.y * 4 + wid) * GEMV_R;
   if (row0 >= W) return;
+  const float bscale = base_gate != nullptr ? sigmoidf_(base_gate[n * bgs]) : 1.0f;
   float acc[GEMV_R];
 #pragma unroll
   for (int r = 0; r < GEMV_R; ++r) acc[r] = 0.0f;
@@ -195,7 +225,7 @@ __global__ __launch_bounds__(256) void expert_down_gemv_kernel(
     const float v = wave_reduce_sum(acc[r]);
     if (lane == 0 && row0 + r < W) {
       const long at = n * W + row0 + r;
-      out[at] = (base != nullptr ? ldf(base + at) : 0.0f) + v;
+      out[at] = (base != nullptr ? ldf(base + at) * bscale : 0.0f) + v;
     }
   }
 }
@@ -220,9 +250,23 @@ static void check_experts(const at::Tensor& h, const at::Tensor& w_up, const at:
   }
 }
 
+// logits of the base row's sigmoid gate: float32, one per token, any stride
+static const float* base_gate_ptr(const c10::optional<at::Tensor>& base_gate, const c10::optional<at::Tensor>& base,
+                                  long N, long* stride) {
+  *stride = 0;
+  if (!base_gate.has_value()) return nullptr;
+  TORCH_CHECK(base.has_value(), "a base gate needs a base");
+  TORCH_CHECK(base_gate->is_cuda() && is_f32(*base_gate) && base_gate->numel() == N && base_gate->dim() <= 2 &&
+              (base_gate->dim() < 2 || base_gate->size(1) == 1), "base_gate must be float32 [N] logits");
+  *stride = N > 0 ? base_gate->stride(0) : 0;
+  return base_gate->data_ptr<float>();
+}
+
 at::Tensor expert_ffn_gemv(at::Tensor h, at::Tensor w_up, at::Tensor w_down, at::Tensor ids, at::Tensor weights,
-                           c10::optional<at::Tensor> base) {
+                           c10::optional<at::Tensor> base, c10::optional<at::Tensor> base_gate) {
   check_experts(h, w_up, w_down, ids, weights, base);
+  long bgs = 0;
+  const float* bgp = base_gate_ptr(base_gate, base, h.size(0), &bgs);
   const long N = h.size(0);
   const int W = (int)h.size(1), E = (int)w_up.size(0), F = (int)w_up.size(1), top = (int)ids.size(1);
   at::Tensor out = at::empty({N, W}, h.options().dtype(at::kFloat));
@@ -242,12 +286,12 @@ at::Tensor expert_ffn_gemv(at::Tensor h, at::Tensor w_up, at::Tensor w_down, at:
       SERVING_DISPATCH_ACT(*base, TB, {
         hipLaunchKernelGGL((expert_down_gemv_kernel<T, TB>), grid, dim3(256), 0, stream(), out.data_ptr<float>(),
                            ptr<T>(hidden), ptr<T>(w_down), ids.data_ptr<int>(), weights.data_ptr<float>(), ptr<TB>(*base),
-                           top, E, F, W, vec_down);
+                           bgp, bgs, top, E, F, W, vec_down);
       });
     } else {
       hipLaunchKernelGGL((expert_down_gemv_kernel<T, float>), grid, dim3(256), 0, stream(), out.data_ptr<float>(),
                          ptr<T>(hidden), ptr<T>(w_down), ids.data_ptr<int>(), weights.data_ptr<float>(),
-                         (const float*)nullptr, top, E, F, W, vec_down);
+                         (const float*)nullptr, (const float*)nullptr, 0L, top, E, F, W, vec_down);
     }
   });
   HIP_CHECK_LAST();
@@ -255,18 +299,21 @@ at::Tensor expert_ffn_gemv(at::Tensor h, at::Tensor w_up, at::Tensor w_down, at:
 }
 
 // ------------------------------------------------------------------ combine
-// out[n, w] = base[n, w] + sum_j weights[n, j] * y[inv[n, j], w], slots in order, float32.
+// out[n, w] = base[n, w] (* sigmoid(base_gate[n])) + sum_j weights[n, j] * y[inv[n, j], w], slots in order, float32.
 // VEC: eight columns per thread (W a multiple of 8, 32-byte aligned operands).
 template <typename T, typename TB, bool VEC>
 __global__ __launch_bounds__(256) void expert_combine_kernel(
     float* __restrict__ out, const T* __restrict__ y, const int* __restrict__ inv, const float* __restrict__ weights,
-    const TB* __restrict__ base, int top, int W, long rows) {
+    const TB* __restrict__ base, const float* __restrict__ base_gate, long bgs, int top, int W, long rows) {
   const long n = blockIdx.x;
+  const float bscale = base_gate != nullptr ? sigmoidf_(base_gate[n * bgs]) : 1.0f;
   if (VEC) {
     for (int w = threadIdx.x * 8; w < W; w += blockDim.x * 8) {
       float acc[8];
       if (base != nullptr) {
         load8(base + n * W + w, acc);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] *= bscale;
       } else {
 #pragma unroll
         for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
@@ -285,7 +332,7 @@ __global__ __launch_bounds__(256) void expert_combine_kernel(
     }
   } else {
     for (int w = threadIdx.x; w < W; w += blockDim.x) {
-      float acc = base != nullptr ? ldf(base + n * W + w) : 0.0f;
+      float acc = base != nullptr ? ldf(base + n * W + w) * bscale : 0.0f;
       for (int j = 0; j < top; ++j) {
         const long r = inv[n * top + j];
         if (r >= 0 && r < rows) acc += weights[n * top + j] * ldf(y + r * W + w);
@@ -295,7 +342,8 @@ __global__ __launch_bounds__(256) void expert_combine_kernel(
   }
 }
 
-at::Tensor expert_combine(at::Tensor y, at::Tensor inv, at::Tensor weights, c10::optional<at::Tensor> base) {
+at::Tensor expert_combine(at::Tensor y, at::Tensor inv, at::Tensor weights, c10::optional<at::Tensor> base,
+                          c10::optional<at::Tensor> base_gate) {
   check_act(y, "y");
   check_i32(inv, "inv");
   TORCH_CHECK(y.dim() == 2 && y.is_contiguous() && inv.dim() == 2 && inv.size(0) * inv.size(1) == y.size(0),
@@ -307,6 +355,8 @@ at::Tensor expert_combine(at::Tensor y, at::Tensor inv, at::Tensor weights, c10:
     check_act(*base, "base");
     TORCH_CHECK(base->is_contiguous() && base->dim() == 2 && base->size(0) == N && base->size(1) == W);
   }
+  long bgs = 0;
+  const float* bgp = base_gate_ptr(base_gate, base, N, &bgs);
   at::Tensor out = at::empty({N, W}, y.options().dtype(at::kFloat));
   if (N == 0) return out;
   auto al32 = [](const at::Tensor& t) { return reinterpret_cast<uintptr_t>(t.data_ptr()) % 32 == 0; };
@@ -316,12 +366,12 @@ at::Tensor expert_combine(at::Tensor y, at::Tensor inv, at::Tensor weights, c10:
   do {                                                                                                                \
     if (vec)                                                                                                          \
       hipLaunchKernelGGL((expert_combine_kernel<T, TB_, true>), dim3((unsigned)N), dim3(256), 0, stream(),           \
-                         out.data_ptr<float>(), ptr<T>(y), inv.data_ptr<int>(), weights.data_ptr<float>(), bp, top, W, \
-                         (long)y.size(0));                                                                            \
+                         out.data_ptr<float>(), ptr<T>(y), inv.data_ptr<int>(), weights.data_ptr<float>(), bp, bgp,  \
+                         bgs, top, W, (long)y.size(0));                                                               \
     else                                                                                                              \
       hipLaunchKernelGGL((expert_combine_kernel<T, TB_, false>), dim3((unsigned)N), dim3(256), 0, stream(),          \
-                         out.data_ptr<float>(), ptr<T>(y), inv.data_ptr<int>(), weights.data_ptr<float>(), bp, top, W, \
-                         (long)y.size(0));                                                                            \
+                         out.data_ptr<float>(), ptr<T>(y), inv.data_ptr<int>(), weights.data_ptr<float>(), bp, bgp,  \
+                         bgs, top, W, (long)y.size(0));                                                               \
   } while (0)
   SERVING_DISPATCH_ACT(y, T, {
     if (base.has_value()) {

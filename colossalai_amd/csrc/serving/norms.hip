@@ -8,7 +8,12 @@
 //                        residual — one pass, the merged row staged in LDS;
 //   add_rms_norm       : residual += a (+ b) in place and, when a weight is
 //                        given, the RMS norm of the new residual row for the
-//                        next pre-norm layer, in one launch.
+//                        next pre-norm layer, in one launch;
+//   gated_grouped_rms_norm : x * silu(gate), then the grouped RMS norm;
+//   add_layer_norm     : centred norm (weight, no bias) of a sublayer's output
+//                        added, scaled, to the residual in place, and the
+//                        centred norm of the new residual row for the next
+//                        sublayer, in one launch.
 #include "serving_common.h"
 
 namespace cai {
@@ -17,25 +22,26 @@ namespace serving {
 // One wave per (row, group).
 template <typename TI, typename TO>
 __global__ __launch_bounds__(256) void grouped_rms_norm_kernel(
-    TO* __restrict__ out, float* __restrict__ residual, const TI* __restrict__ x, const float* __restrict__ w,
+    TO* __restrict__ out, float* __restrict__ residual, const TI* __restrict__ x, long xs, const float* __restrict__ w,
     long units, int groups, int gs, float eps) {
   const int lane = threadIdx.x & 63;
   const long unit = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   if (unit >= units) return;
   const long row = unit / groups;
   const int g = (int)(unit % groups);
-  const long base = (row * groups + g) * (long)gs;
+  const long base = (row * groups + g) * (long)gs;   // in the dense output / residual
+  const TI* xr = x + row * xs + (long)g * gs;        // the input's rows may be strided
   float ssq = 0.0f;
 #pragma unroll 8
   for (int i = lane; i < gs; i += 64) {  // unrolled: the loads of a row are in flight together
-    const float v = ldf(x + base + i);
+    const float v = ldf(xr + i);
     ssq += v * v;
   }
   ssq = wave_reduce_sum(ssq);
   const float inv = 1.0f / sqrtf(ssq / (float)gs + eps);
 #pragma unroll 8
   for (int i = lane; i < gs; i += 64) {
-    const float y = ldf(x + base + i) * inv * w[g * gs + i];
+    const float y = ldf(xr + i) * inv * w[g * gs + i];
     if (residual != nullptr) residual[base + i] += y;
     else stf(out + base + i, y);
   }
@@ -44,17 +50,18 @@ __global__ __launch_bounds__(256) void grouped_rms_norm_kernel(
 at::Tensor grouped_rms_norm(at::Tensor x, at::Tensor weight, int64_t groups, double eps,
                             c10::optional<at::Tensor> residual, at::ScalarType out_dtype) {
   check_act(x, "x");
-  TORCH_CHECK(x.dim() == 2 && x.is_contiguous(), "x must be contiguous [N, W]");
+  TORCH_CHECK(x.dim() == 2 && x.stride(1) == 1, "x must be [N, W] with unit inner stride");
   const long N = x.size(0);
   const int W = (int)x.size(1);
+  const long xs = x.stride(0);
   TORCH_CHECK(groups > 0 && W % groups == 0);
   at::Tensor w = f32c(weight);
   TORCH_CHECK(w.numel() == W);
   float* res = nullptr;
   at::Tensor out;
   if (residual.has_value()) {
-    TORCH_CHECK(is_f32(*residual) && residual->is_contiguous() && residual->sizes() == x.sizes(),
-                "residual must be contiguous float32 of x's shape");
+    TORCH_CHECK(is_f32(*residual) && residual->is_contiguous() && residual->sizes() == x.sizes() && x.is_contiguous(),
+                "residual must be contiguous float32 of x's shape, and x contiguous with it");
     res = residual->data_ptr<float>();
     out = *residual;
   } else {
@@ -66,11 +73,11 @@ at::Tensor grouped_rms_norm(at::Tensor x, at::Tensor weight, int64_t groups, dou
   SERVING_DISPATCH_ACT(x, TI, {
     if (res != nullptr) {
       hipLaunchKernelGGL((grouped_rms_norm_kernel<TI, float>), dim3(grid), dim3(256), 0, stream(), (float*)nullptr, res,
-                         ptr<TI>(x), w.data_ptr<float>(), units, (int)groups, W / (int)groups, (float)eps);
+                         ptr<TI>(x), xs, w.data_ptr<float>(), units, (int)groups, W / (int)groups, (float)eps);
     } else {
       SERVING_DISPATCH_ACT(out, TO, {
         hipLaunchKernelGGL((grouped_rms_norm_kernel<TI, TO>), dim3(grid), dim3(256), 0, stream(), ptr<TO>(out),
-                           (float*)nullptr, ptr<TI>(x), w.data_ptr<float>(), units, (int)groups, W / (int)groups,
+                           (float*)nullptr, ptr<TI>(x), xs, w.data_ptr<float>(), units, (int)groups, W / (int)groups,
                            (float)eps);
       });
     }
@@ -322,6 +329,233 @@ c10::optional<at::Tensor> add_rms_norm(at::Tensor residual, at::Tensor a, c10::o
     HIP_CHECK_LAST();
   }
   if (!weight.has_value()) return c10::nullopt;
+  return out;
+}
+
+// ------------------------------------------------------- gate, then grouped RMS norm
+// One wave per (row, group): out = rms_unit(x * silu(gate)) * w over the group. x dense [N, W]
+// (float32 or an activation type), gate row-strided.
+template <typename TX, typename TG, typename TO>
+__global__ __launch_bounds__(256) void gated_grouped_rms_norm_kernel(
+    TO* __restrict__ out, const TX* __restrict__ x, const TG* __restrict__ gate, long gstride,
+    const float* __restrict__ w, long units, int groups, int gs, float eps) {
+  const int lane = threadIdx.x & 63;
+  const long unit = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (unit >= units) return;
+  const long row = unit / groups;
+  const int g = (int)(unit % groups);
+  const long base = (row * groups + g) * (long)gs;
+  const TG* gr = gate + row * gstride + (long)g * gs;
+  float ssq = 0.0f;
+#pragma unroll 4
+  for (int i = lane; i < gs; i += 64) {
+    const float z = ldf(gr + i);
+    const float v = ldf(x + base + i) * (z * sigmoidf_(z));
+    ssq += v * v;
+  }
+  ssq = wave_reduce_sum(ssq);
+  const float inv = 1.0f / sqrtf(ssq / (float)gs + eps);
+#pragma unroll 4
+  for (int i = lane; i < gs; i += 64) {
+    const float z = ldf(gr + i);
+    stf(out + base + i, ldf(x + base + i) * (z * sigmoidf_(z)) * inv * w[g * gs + i]);
+  }
+}
+
+at::Tensor gated_grouped_rms_norm(at::Tensor x, at::Tensor gate, at::Tensor weight, int64_t groups, double eps,
+                                  at::ScalarType out_dtype) {
+  check_act(x, "x"); check_act(gate, "gate");
+  TORCH_CHECK(x.dim() == 2 && x.is_contiguous(), "x must be contiguous [N, W]");
+  TORCH_CHECK(gate.dim() == 2 && gate.sizes() == x.sizes() && gate.stride(1) == 1, "gate must be [N, W] with unit inner stride");
+  const long N = x.size(0);
+  const int W = (int)x.size(1);
+  TORCH_CHECK(groups > 0 && W % groups == 0);
+  at::Tensor w = f32c(weight);
+  TORCH_CHECK(w.numel() == W);
+  at::Tensor out = at::empty({N, W}, x.options().dtype(out_dtype));
+  check_act(out, "out");
+  if (N == 0) return out;
+  const long units = N * groups;
+  const unsigned grid = (unsigned)((units + 3) / 4);
+  SERVING_DISPATCH_ACT(x, TX, {
+    SERVING_DISPATCH_ACT(gate, TG, {
+      SERVING_DISPATCH_ACT(out, TO, {
+        hipLaunchKernelGGL((gated_grouped_rms_norm_kernel<TX, TG, TO>), dim3(grid), dim3(256), 0, stream(), ptr<TO>(out),
+                           ptr<TX>(x), ptr<TG>(gate), (long)gate.stride(0), w.data_ptr<float>(), units, (int)groups,
+                           W / (int)groups, (float)eps);
+      });
+    });
+  });
+  HIP_CHECK_LAST();
+  return out;
+}
+
+// ------------------------------------------------- centred norm on the way in and out
+// One block per row. With a residual: residual += mult * layer_norm(y) * w_out in place; then, with
+// w_next, out = layer_norm(residual) * w_next. Without a residual: out = layer_norm(y) * w_next.
+// layer_norm(v) = (v - mean) / sqrt(mean((v - mean)^2) + eps): the variance is taken from the
+// deviations (a second pass over registers), not from the mean of squares.
+// CH > 0: each thread owns CH chunks of 8 consecutive elements in registers (W a multiple of 8 up to
+// 2048 * CH, aligned operands), every operand is read once with 16/32-byte loads. CH == 0: any W,
+// the row is staged in LDS.
+template <typename TY, typename TO, int CH>
+__global__ __launch_bounds__(256) void add_layer_norm_kernel(
+    TO* __restrict__ out, float* __restrict__ residual, const TY* __restrict__ y, const float* __restrict__ w_out,
+    float mult, const float* __restrict__ w_next, int W, float eps) {
+  __shared__ float red[8];
+  extern __shared__ __align__(16) float rowbuf[];
+  const long row = blockIdx.x;
+  const float invW = 1.0f / (float)W;
+  if constexpr (CH > 0) {
+    float r[CH][8];
+    float sum = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int i = (threadIdx.x + 256 * c) * 8;
+      if (i < W) {
+        load8(y + row * W + i, r[c]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sum += r[c][e];
+      }
+    }
+    if (residual != nullptr) {
+      const float mean = block_reduce_sum(sum, red) * invW;
+      float ssq = 0.0f;
+#pragma unroll
+      for (int c = 0; c < CH; ++c)
+        if ((threadIdx.x + 256 * c) * 8 < W) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            r[c][e] -= mean;
+            ssq += r[c][e] * r[c][e];
+          }
+        }
+      const float inv = mult / sqrtf(block_reduce_sum(ssq, red) * invW + eps);
+      sum = 0.0f;
+#pragma unroll
+      for (int c = 0; c < CH; ++c) {
+        const int i = (threadIdx.x + 256 * c) * 8;
+        if (i < W) {
+          float wv[8], xv[8];
+          load8(w_out + i, wv);
+          load8(residual + row * W + i, xv);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            r[c][e] = xv[e] + r[c][e] * inv * wv[e];
+            sum += r[c][e];
+          }
+          store8(residual + row * W + i, r[c]);
+        }
+      }
+      if (w_next == nullptr) return;
+    }
+    const float mean = block_reduce_sum(sum, red) * invW;
+    float ssq = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c)
+      if ((threadIdx.x + 256 * c) * 8 < W) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          r[c][e] -= mean;
+          ssq += r[c][e] * r[c][e];
+        }
+      }
+    const float inv = 1.0f / sqrtf(block_reduce_sum(ssq, red) * invW + eps);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int i = (threadIdx.x + 256 * c) * 8;
+      if (i < W) {
+        float wv[8];
+        load8(w_next + i, wv);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) wv[e] *= r[c][e] * inv;
+        store8(out + row * W + i, wv);
+      }
+    }
+  } else {
+    float sum = 0.0f;
+    for (int i = threadIdx.x; i < W; i += blockDim.x) {
+      const float v = ldf(y + row * W + i);
+      rowbuf[i] = v;
+      sum += v;
+    }
+    if (residual != nullptr) {
+      const float mean = block_reduce_sum(sum, red) * invW;
+      float ssq = 0.0f;
+      for (int i = threadIdx.x; i < W; i += blockDim.x) {
+        const float d = rowbuf[i] - mean;
+        ssq += d * d;
+      }
+      const float inv = mult / sqrtf(block_reduce_sum(ssq, red) * invW + eps);
+      sum = 0.0f;
+      for (int i = threadIdx.x; i < W; i += blockDim.x) {
+        const float v = residual[row * W + i] + (rowbuf[i] - mean) * inv * w_out[i];
+        residual[row * W + i] = v;
+        rowbuf[i] = v;
+        sum += v;
+      }
+      if (w_next == nullptr) return;
+    }
+    const float mean = block_reduce_sum(sum, red) * invW;
+    float ssq = 0.0f;
+    for (int i = threadIdx.x; i < W; i += blockDim.x) {
+      const float d = rowbuf[i] - mean;
+      ssq += d * d;
+    }
+    const float inv = 1.0f / sqrtf(block_reduce_sum(ssq, red) * invW + eps);
+    for (int i = threadIdx.x; i < W; i += blockDim.x) stf(out + row * W + i, (rowbuf[i] - mean) * inv * w_next[i]);
+  }
+}
+
+c10::optional<at::Tensor> add_layer_norm(c10::optional<at::Tensor> residual, at::Tensor y,
+                                         c10::optional<at::Tensor> w_out, double mult,
+                                         c10::optional<at::Tensor> w_next, double eps, at::ScalarType out_dtype) {
+  check_act(y, "y");
+  TORCH_CHECK(y.dim() == 2 && y.is_contiguous(), "y must be contiguous [N, W]");
+  const long N = y.size(0);
+  const int W = (int)y.size(1);
+  TORCH_CHECK(residual.has_value() == w_out.has_value(), "a residual needs the weight of the norm on its way in");
+  TORCH_CHECK(residual.has_value() || w_next.has_value(), "nothing to compute");
+  float* rp = nullptr;
+  at::Tensor wo, wn, out;
+  const float *wop = nullptr, *wnp = nullptr;
+  if (residual.has_value()) {
+    TORCH_CHECK(residual->is_cuda() && is_f32(*residual) && residual->is_contiguous() && residual->sizes() == y.sizes(),
+                "residual must be contiguous float32 of y's shape");
+    rp = residual->data_ptr<float>();
+    wo = f32c(*w_out);
+    TORCH_CHECK(wo.numel() == W);
+    wop = wo.data_ptr<float>();
+  }
+  if (w_next.has_value()) {
+    wn = f32c(*w_next);
+    TORCH_CHECK(wn.numel() == W);
+    wnp = wn.data_ptr<float>();
+    out = at::empty({N, W}, y.options().dtype(out_dtype));
+    check_act(out, "out");
+  }
+  if (N > 0) {
+    const at::Tensor& like = w_next.has_value() ? out : y;   // without w_next nothing is written through `out`
+    auto al32 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 32 == 0; };
+    const bool rows = W % 8 == 0 && W <= 2048 * 4 && al32(y.data_ptr()) && (rp == nullptr || (al32(rp) && al32(wop))) &&
+                      (wnp == nullptr || (al32(wnp) && al32(out.data_ptr())));
+    TORCH_CHECK(rows || (size_t)W * sizeof(float) <= 64 * 1024, "row too long for the norm kernel");
+#define LN_LAUNCH(CH_, SMEM_)                                                                                      \
+  hipLaunchKernelGGL((add_layer_norm_kernel<TY, TO, CH_>), dim3((unsigned)N), dim3(256), SMEM_, stream(), op, rp, \
+                     ptr<TY>(y), wop, (float)mult, wnp, W, (float)eps)
+    SERVING_DISPATCH_ACT(y, TY, {
+      SERVING_DISPATCH_ACT(like, TO, {
+        TO* op = w_next.has_value() ? ptr<TO>(out) : (TO*)nullptr;
+        if (rows && W <= 2048) LN_LAUNCH(1, 0);
+        else if (rows && W <= 4096) LN_LAUNCH(2, 0);
+        else if (rows) LN_LAUNCH(4, 0);
+        else LN_LAUNCH(0, (size_t)W * sizeof(float));
+      });
+    });
+#undef LN_LAUNCH
+    HIP_CHECK_LAST();
+  }
+  if (!w_next.has_value()) return c10::nullopt;
   return out;
 }
 

@@ -50,7 +50,9 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
     const T* __restrict__ vpool, const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ tok_seq,
     const int* __restrict__ positions, const float* __restrict__ slopes, const T* __restrict__ gate, long gate_stride,
     int H, int G, int D, int Dv, int page_shift, float scale, int window, int keep_first, int kvec, int vvec,
-    float softcap, int sink) {
+    float softcap, int sink, long vrow, long vhead) {
+  // vrow / vhead: elements between the value rows of neighbouring pool rows / kv heads (G * Dv and Dv for a
+  // pool of its own; a value pool that is a view into wider rows, e.g. the leading channels of the keys, has others)
   extern __shared__ __align__(16) float lds[];
   const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
   const int Dp = (D + 7) & ~7;
@@ -169,7 +171,7 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
 #pragma unroll 4
       for (int jj = vsub; jj < cnt; jj += vks) {
         float v[8];
-        load8(vpool + ((long)prow[jj] * G + g) * Dv + vch, v);
+        load8(vpool + (long)prow[jj] * vrow + (long)g * vhead + vch, v);
 #pragma unroll
         for (int r = 0; r < RC; ++r) {
           const float w = pw[r * 64 + jj];
@@ -181,7 +183,7 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
     const int dva = 2 * lane, dvb = 128 + 2 * lane;
 #pragma unroll 8
     for (int jj = 0; jj < cnt; ++jj) {
-      const T* vr = vpool + ((long)prow[jj] * G + g) * Dv;
+      const T* vr = vpool + (long)prow[jj] * vrow + (long)g * vhead;
       float v0 = 0.0f, v1 = 0.0f, v2 = 0.0f, v3 = 0.0f;
       if (vvec) {
         if (dva < Dv) load2(vr + dva, v0, v1);
@@ -534,14 +536,18 @@ at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at:
   check_act(q, "q");
   TORCH_CHECK(softcap >= 0.0, "softcap must not be negative (0 = none)");
   TORCH_CHECK(q.dim() == 3 && q.stride(2) == 1 && q.stride(1) == q.size(2), "q must be [N, H, D] with dense rows");
-  TORCH_CHECK(kpool.dim() == 4 && vpool.dim() == 4 && kpool.is_contiguous() && vpool.is_contiguous());
+  // the value pool may be a view into wider rows (values that are leading channels of the keys): dense
+  // channels, pages of `page` rows, any row and head stride
+  TORCH_CHECK(kpool.dim() == 4 && vpool.dim() == 4 && kpool.is_contiguous() && vpool.stride(3) == 1 &&
+              vpool.stride(0) == vpool.size(1) * vpool.stride(1), "pools must be [pages, page, G, D] with dense rows");
   TORCH_CHECK(kpool.scalar_type() == q.scalar_type() && vpool.scalar_type() == q.scalar_type(),
               "query and pools share one dtype");
   const long N = q.size(0);
   const int H = (int)q.size(1), D = (int)q.size(2);
   const int page = (int)kpool.size(1), G = (int)kpool.size(2), Dv = (int)vpool.size(3);
   TORCH_CHECK(kpool.size(3) == D && vpool.size(2) == G && vpool.size(1) == page && vpool.size(0) == kpool.size(0));
-  TORCH_CHECK(H % G == 0 && Dv <= 256 && page > 0 && (page & (page - 1)) == 0);
+  TORCH_CHECK(H % G == 0 && Dv <= 512 && page > 0 && (page & (page - 1)) == 0);
+  const long vrow = vpool.stride(1), vhead = G > 1 ? vpool.stride(2) : Dv;
   check_i32(block_tables, "block_tables"); check_i32(tok_seq, "tok_seq"); check_i32(positions, "positions");
   TORCH_CHECK(block_tables.dim() == 2 && tok_seq.numel() == N && positions.numel() == N);
   TORCH_CHECK(window >= 0 && keep_first >= 0);
@@ -568,7 +574,7 @@ at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at:
   const bool aligned = q.stride(0) % 8 == 0 && reinterpret_cast<uintptr_t>(q.data_ptr()) % 16 == 0;
   // head sizes that are multiples of 8 ride in the next larger tiling, zero-padded
   const bool mfma_shape = D % 8 == 0 && Dv % 8 == 0 && D <= 128 && Dv <= 128;
-  if (num_tiles > 0 && is_bf16(q) && aligned && mfma_shape) {
+  if (num_tiles > 0 && is_bf16(q) && aligned && mfma_shape && vpool.is_contiguous()) {
     const int rep = H / G, nw = 4;
     const dim3 grid((unsigned)num_tiles, (unsigned)G, (unsigned)((rep + nw - 1) / nw));
     const int ds = D <= 32 ? 2 : D <= 48 ? 3 : D <= 64 ? 4 : D <= 96 ? 6 : 8, vt = (Dv + 31) / 32;
@@ -605,15 +611,21 @@ at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at:
   const int R = H / G;
   int rc = RC_MAX;
   while (rc > 1 && (rc > R || N * G * ((R + rc - 1) / rc) < 256)) rc >>= 1;  // enough blocks to cover the CUs
-  const int chunks = (R + rc - 1) / rc;
   auto lds_bytes = [&](int nw) { return (size_t)(rc * Dp + nw * (rc * 64 + 64) + nw * rc * (2 + Dv)) * sizeof(float); };
-  const int nwaves = lds_bytes(ATT_WAVES) <= 64 * 1024 ? ATT_WAVES : ATT_WAVES / 2;
+  // wide value rows (a latent of several hundred channels): fewer waves, then fewer heads per block
+  int nwaves = ATT_WAVES;
+  while (lds_bytes(nwaves) > 64 * 1024 && nwaves > 4) nwaves >>= 1;
+  while (lds_bytes(nwaves) > 64 * 1024 && rc > 1) rc >>= 1;
+  const int chunks = (R + rc - 1) / rc;
   const size_t smem = lds_bytes(nwaves);
   TORCH_CHECK(smem <= 64 * 1024, "head sizes too large for the scalar attention kernel");
   const int kvec = D % 8 == 0 ? 1 : 0;   // 16-byte (bfloat16) / 32-byte (float32) aligned key slices
-  const int vvec = Dv % 2 == 0 ? 1 : 0;
+  const int vvec_even = Dv % 2 == 0 ? 1 : 0;
   // value rows of 8, 16, ..., 256 channels whose loads are aligned take the 8-channels-per-lane value phase
-  const bool v8 = Dv >= 8 && (Dv & (Dv - 1)) == 0 && reinterpret_cast<uintptr_t>(vpool.data_ptr()) % 32 == 0;
+  const bool v8 = Dv >= 8 && (Dv & (Dv - 1)) == 0 && reinterpret_cast<uintptr_t>(vpool.data_ptr()) % 32 == 0 &&
+                  vrow % 8 == 0 && vhead % 8 == 0;
+  TORCH_CHECK(v8 || Dv <= 256, "value rows above 256 channels must be a power of two and aligned");
+  const int vvec_ok = (vrow % 2 == 0 && vhead % 2 == 0) ? 1 : 0;
 #define SCALAR_CASE(RC_)                                                                                            \
   if (v8) SCALAR_LAUNCH(RC_, true);                                                                                 \
   else SCALAR_LAUNCH(RC_, false)
@@ -622,8 +634,8 @@ at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at:
                      stream(), ptr<T>(out), ptr<T>(q), (long)q.stride(0), ptr<T>(kpool), ptr<T>(vpool),             \
                      block_tables.data_ptr<int>(), (int)block_tables.stride(0), tok_seq.data_ptr<int>(),            \
                      positions.data_ptr<int>(), slp, gate.has_value() ? ptr<T>(*gate) : (const T*)nullptr, gstride, \
-                     H, G, D, Dv, page_shift, (float)scale, (int)window, (int)keep_first, kvec, vvec,                \
-                     (float)softcap, sink ? 1 : 0)
+                     H, G, D, Dv, page_shift, (float)scale, (int)window, (int)keep_first, kvec,                      \
+                     vvec_even & vvec_ok, (float)softcap, sink ? 1 : 0, vrow, vhead)
   SERVING_DISPATCH_ACT(q, T, {
     if (rc == 4) { SCALAR_CASE(4); }
     else if (rc == 2) { SCALAR_CASE(2); }

@@ -7,7 +7,11 @@ namespace cai {
 namespace serving {
 
 at::Tensor short_conv(at::Tensor x, at::Tensor taps, c10::optional<at::Tensor> tail, at::Tensor cu, at::Tensor start,
-                      at::Tensor slots, at::Tensor tok_seq, bool silu, at::ScalarType out_dtype);
+                      at::Tensor slots, at::Tensor tok_seq, bool silu, at::ScalarType out_dtype,
+                      c10::optional<at::Tensor> bias);
+at::Tensor ssd_recurrence(at::Tensor x, at::Tensor Bm, at::Tensor Cm, at::Tensor dt_raw, at::Tensor A_log,
+                          at::Tensor dt_bias, at::Tensor D_skip, at::Tensor state, at::Tensor cu, at::Tensor start,
+                          at::Tensor slots);
 at::Tensor gated_delta_rule(at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor beta_logit, at::Tensor dt,
                             at::Tensor A_log, at::Tensor dt_bias, at::Tensor state, at::Tensor cu, at::Tensor start,
                             at::Tensor slots, double unit_eps, double q_scale);
@@ -19,7 +23,8 @@ at::Tensor tied_gate_recurrence(at::Tensor q, at::Tensor f_logit, at::Tensor v, 
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   namespace s = cai::serving;
-  m.def("short_conv", &s::short_conv, "short causal depthwise convolution with carried tail");
+  m.def("short_conv", &s::short_conv, "short causal depthwise convolution with carried tail and optional bias");
+  m.def("ssd_recurrence", &s::ssd_recurrence, "state-space recurrence with one decay per head, carried state");
   m.def("gated_delta_rule", &s::gated_delta_rule, "gated delta rule with per-channel decay, carried state");
   m.def("tied_gate_recurrence", &s::tied_gate_recurrence, "HGRN2-style recurrence, carried state");
 }

@@ -11,6 +11,7 @@
 //
 //   delta: S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q
 //   tied : S <- diag(f) S + (1 - f) v^T;                          o = S^T q
+//   ssd  : S <- a S + (dt v) k^T  (one decay a per head and token);   o = S^T q + D_skip v
 //
 // A prologue kernel turns the raw projections into float32 operands once per
 // token (unit-length q/k, decay from its logits, gates), so the sequential
@@ -67,6 +68,20 @@ __global__ __launch_bounds__(256) void tied_prepare_kernel(
   }
 }
 
+// scal[n, h] = (a, dt): dt = softplus(dt_raw + dt_bias) (no clamp), a = exp(-exp(A_log) dt).
+template <typename TL>
+__global__ __launch_bounds__(256) void ssd_prepare_kernel(float* __restrict__ scal, const TL* __restrict__ dt, long ds,
+                                                          const float* __restrict__ A_log,
+                                                          const float* __restrict__ dt_bias, long N, int H) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= N * H) return;
+  const long n = i / H;
+  const int h = (int)(i % H);
+  const float d = softplusf_(ldf(dt + n * ds + h) + dt_bias[h]);
+  scal[2 * i] = expf(-expf(A_log[h]) * d);
+  scal[2 * i + 1] = d;
+}
+
 // ---------------------------------------------------------------------- scan
 // Sum over the P adjacent lanes that share a value channel, on the DPP path
 // (no LDS traffic): xor 1 and 2 inside a quad, then the half-row and row
@@ -94,15 +109,22 @@ DEV_INLINE float reduce_p(float v) {
 // prompt (D = 128): NC = 2 is 1.5x slower per layer than NC = 1 - a single long sequence is
 // bound by the instructions a wave issues per token, not by latencies that a second chain could
 // hide - so NC stays 1.
-template <int P, int DPL, bool DELTA, typename TV>
+// MODE: 0 = tied, 1 = delta, 2 = ssd. In ssd mode the operand rows are q and k (no per-channel gate) with the
+// token stride qk_ts, `beta` holds two scalars per (token, head), the decay a and the step dt, and `skip` [H] the
+// weight of the direct path.
+constexpr int SCAN_TIED = 0, SCAN_DELTA = 1, SCAN_SSD = 2;
+
+template <int P, int DPL, int MODE, typename TV>
 __global__ __launch_bounds__(256) void matrix_state_scan_kernel(
     float* __restrict__ out, const float* __restrict__ q, const float* __restrict__ k, const float* __restrict__ gate,
     const float* __restrict__ beta, const TV* __restrict__ v, long vs, float* __restrict__ state, long ss,
     const int* __restrict__ cu, const int* __restrict__ start, const int* __restrict__ slots, int H, int rep, int D,
-    int Dv) {
+    int Dv, long qk_ts, int vec_ok, const float* __restrict__ skip) {
+  constexpr bool DELTA = MODE == SCAN_DELTA, SSD = MODE == SCAN_SSD;
   constexpr int Dp = P * DPL;                 // padded key size
   constexpr int CT = Dp > 128 ? 8 : 16;       // tokens per staged chunk
-  constexpr int NOPS = DELTA ? 3 : 2;         // q, (k,) gate
+  constexpr int NOPS = DELTA ? 3 : 2;         // q, (k,) gate; ssd: q, k
+  constexpr int NB = SSD ? 2 : 1;             // scalars per (token, head)
   constexpr int NC = 1;                       // value channels per lane
   constexpr int CPW = 4 * 64 / P;             // lanes groups (one channel each) per block
   constexpr int CPB = CPW * NC;               // value channels per block
@@ -111,7 +133,7 @@ __global__ __launch_bounds__(256) void matrix_state_scan_kernel(
   extern __shared__ __align__(16) float lds[];
   float* ops_buf = lds;                       // [2][CT][NOPS][Dp]
   float* v_buf = lds + 2 * OPF;               // [2][CT][CPB]
-  float* b_buf = v_buf + 2 * CT * CPB;        // [2][CT]
+  float* b_buf = v_buf + 2 * CT * CPB;        // [2][CT][NB]
 
   const int b = blockIdx.z, h = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6;
@@ -141,11 +163,12 @@ __global__ __launch_bounds__(256) void matrix_state_scan_kernel(
   constexpr int RF4 = Dp / 4, OPF4 = CT * NOPS * RF4, R_OP4 = (OPF4 + 255) / 256;
   float4v r_op[R_OP4];
   float r_v[R_V], r_b = 0.0f;
-  const bool rows_vec = (D % 4) == 0;
+  const bool rows_vec = (D % 4) == 0 && vec_ok;
   const float* q_head = q + (long)hq * D;
-  const float* k_head = DELTA ? k + (long)hq * D : nullptr;
-  const float* g_head = gate + (long)h * D;
-  const long qk_stride = (long)Hq * D, g_stride = (long)H * D;
+  const float* k_head = (DELTA || SSD) ? k + (long)hq * D : nullptr;
+  const float* g_head = SSD ? nullptr : gate + (long)h * D;
+  const long qk_stride = SSD ? qk_ts : (long)Hq * D, g_stride = (long)H * D;
+  const float dskip = SSD ? skip[h] : 0.0f;
   auto fetch = [&](int tb) {  // chunk starting at token tb -> registers
 #pragma unroll
     for (int r = 0; r < R_OP4; ++r) {
@@ -153,10 +176,11 @@ __global__ __launch_bounds__(256) void matrix_state_scan_kernel(
       const int rowi = i / RF4, f4 = i % RF4;
       const int tok = rowi / NOPS, op = rowi % NOPS;
       const int t = tb + tok, d = f4 * 4;
-      const float fill = (op == NOPS - 1) ? 1.0f : 0.0f;
+      const bool is_gate = !SSD && op == NOPS - 1;
+      const float fill = is_gate ? 1.0f : 0.0f;
       float4v val = {fill, fill, fill, fill};
       if (i < OPF4 && t < t1 && d < D) {
-        const float* src = (op == NOPS - 1) ? g_head + t * g_stride : ((op == 0) ? q_head : k_head) + t * qk_stride;
+        const float* src = is_gate ? g_head + t * g_stride : ((op == 0) ? q_head : k_head) + t * qk_stride;
         if (rows_vec) {
           val = *reinterpret_cast<const float4v*>(src + d);
         } else {
@@ -175,6 +199,7 @@ __global__ __launch_bounds__(256) void matrix_state_scan_kernel(
       r_v[r] = (i < CT * CPB && t < t1) ? ldf(v + (long)t * vs + (long)h * Dv + ch) : 0.0f;
     }
     if (DELTA) r_b = (tid < CT && tb + tid < t1) ? beta[(long)(tb + tid) * H + h] : 0.0f;
+    if (SSD) r_b = (tid < 2 * CT && tb + tid / 2 < t1) ? beta[((long)(tb + tid / 2) * H + h) * 2 + (tid & 1)] : 0.0f;
   };
   auto stash = [&](int buf) {  // registers -> LDS buffer ([CT][NOPS][Dp], the order the rows were fetched in)
 #pragma unroll
@@ -187,7 +212,7 @@ __global__ __launch_bounds__(256) void matrix_state_scan_kernel(
       const int i = tid + 256 * r;
       if (i < CT * CPB) v_buf[buf * CT * CPB + i] = r_v[r];
     }
-    if (DELTA && tid < CT) b_buf[buf * CT + tid] = r_b;
+    if ((DELTA || SSD) && tid < NB * CT) b_buf[buf * NB * CT + tid] = r_b;
   };
 
   fetch(t0);
@@ -205,14 +230,17 @@ __global__ __launch_bounds__(256) void matrix_state_scan_kernel(
       for (int j = 0; j < DPL; j += 4) {
         const float4v a = *reinterpret_cast<const float4v*>(row + j);
         qc[j] = a[0]; qc[j + 1] = a[1]; qc[j + 2] = a[2]; qc[j + 3] = a[3];
-        if (DELTA) {
+        if (DELTA || SSD) {
           const float4v kk = *reinterpret_cast<const float4v*>(row + Dp + j);
           kc[j] = kk[0]; kc[j + 1] = kk[1]; kc[j + 2] = kk[2]; kc[j + 3] = kk[3];
         }
-        const float4v gg = *reinterpret_cast<const float4v*>(row + (NOPS - 1) * Dp + j);
-        gc[j] = gg[0]; gc[j + 1] = gg[1]; gc[j + 2] = gg[2]; gc[j + 3] = gg[3];
+        if (!SSD) {
+          const float4v gg = *reinterpret_cast<const float4v*>(row + (NOPS - 1) * Dp + j);
+          gc[j] = gg[0]; gc[j + 1] = gg[1]; gc[j + 2] = gg[2]; gc[j + 3] = gg[3];
+        }
       }
-      const float bc = DELTA ? b_buf[buf * CT + tt] : 0.0f;
+      const float bc = (DELTA || SSD) ? b_buf[(buf * CT + tt) * NB] : 0.0f;         // delta: beta; ssd: the decay a
+      const float dtc = SSD ? b_buf[(buf * CT + tt) * NB + 1] : 0.0f;               // ssd: the step dt
 #pragma unroll
       for (int x = 0; x < NC; ++x) {
         const float vc = v_buf[buf * CT * CPB + tt * CPB + x * CPW + cl];
@@ -235,6 +263,15 @@ __global__ __launch_bounds__(256) void matrix_state_scan_kernel(
             oa += S[x][j] * qc[j];
             ob += S[x][j + 1] * qc[j + 1];
           }
+        } else if (SSD) {
+          const float xv = dtc * vc;
+#pragma unroll
+          for (int j = 0; j < DPL; j += 2) {
+            S[x][j] = bc * S[x][j] + kc[j] * xv;
+            S[x][j + 1] = bc * S[x][j + 1] + kc[j + 1] * xv;
+            oa += S[x][j] * qc[j];
+            ob += S[x][j + 1] * qc[j + 1];
+          }
         } else {
 #pragma unroll
           for (int j = 0; j < DPL; j += 2) {
@@ -244,7 +281,7 @@ __global__ __launch_bounds__(256) void matrix_state_scan_kernel(
             ob += S[x][j + 1] * qc[j + 1];
           }
         }
-        const float o = reduce_p<P>(oa + ob);
+        const float o = reduce_p<P>(oa + ob) + dskip * vc;
         if (p == 0 && live[x]) out[((long)(tb + tt) * H + h) * Dv + c[x]] = o;
       }
     }
@@ -260,20 +297,21 @@ __global__ __launch_bounds__(256) void matrix_state_scan_kernel(
     }
 }
 
-template <bool DELTA, typename TV>
+template <int MODE, typename TV>
 static void launch_scan(float* out, const float* q, const float* k, const float* gate, const float* beta, const TV* v,
                         long vs, float* state, long ss, const int* cu, const int* start, const int* slots, int B,
-                        int H, int rep, int D, int Dv) {
+                        int H, int rep, int D, int Dv, long qk_ts = 0, int vec_ok = 1, const float* skip = nullptr) {
+  constexpr bool DELTA = MODE == SCAN_DELTA;
   TORCH_CHECK(D <= 256, "key size above 256 is not supported by the recurrence kernel");
   const int dpl = D > 128 ? 16 : 8;
   int P = 1;
   while (P * dpl < D) P <<= 1;
   const int cpb = 4 * 64 / P /* times NC of the kernel */, Dp = P * dpl, ct = Dp > 128 ? 8 : 16, nops = DELTA ? 3 : 2;
   const dim3 grid((unsigned)((Dv + cpb - 1) / cpb), (unsigned)H, (unsigned)B);
-  const size_t smem = (size_t)(2 * ct * nops * Dp + 2 * ct * cpb + 2 * ct) * sizeof(float);
+  const size_t smem = (size_t)(2 * ct * nops * Dp + 2 * ct * cpb + 4 * ct) * sizeof(float);
 #define SCAN_CASE(PP, DD)                                                                                          \
-  hipLaunchKernelGGL((matrix_state_scan_kernel<PP, DD, DELTA, TV>), grid, dim3(256), smem, stream(), out, q, k,   \
-                     gate, beta, v, vs, state, ss, cu, start, slots, H, rep, D, Dv)
+  hipLaunchKernelGGL((matrix_state_scan_kernel<PP, DD, MODE, TV>), grid, dim3(256), smem, stream(), out, q, k,    \
+                     gate, beta, v, vs, state, ss, cu, start, slots, H, rep, D, Dv, qk_ts, vec_ok, skip)
   if (dpl == 16) SCAN_CASE(16, 16);
   else if (P == 1) SCAN_CASE(1, 8);
   else if (P == 2) SCAN_CASE(2, 8);
@@ -326,7 +364,7 @@ at::Tensor gated_delta_rule(at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor
                          bf.data_ptr<float>(), G, H, D, (float)unit_eps, (float)q_scale);
     });
     HIP_CHECK_LAST();
-    launch_scan<true, T>(out.data_ptr<float>(), qn.data_ptr<float>(), kn.data_ptr<float>(), dec.data_ptr<float>(),
+    launch_scan<SCAN_DELTA, T>(out.data_ptr<float>(), qn.data_ptr<float>(), kn.data_ptr<float>(), dec.data_ptr<float>(),
                          beta.data_ptr<float>(), ptr<T>(v), (long)v.stride(0), state.data_ptr<float>(),
                          (long)state.stride(0), cu.data_ptr<int>(), start.data_ptr<int>(), slots.data_ptr<int>(), B, H,
                          H / G, D, Dv);
@@ -355,10 +393,51 @@ at::Tensor tied_gate_recurrence(at::Tensor q, at::Tensor f_logit, at::Tensor v, 
                        f.data_ptr<float>(), ptr<T>(q), (long)q.stride(0), ptr<T>(f_logit), (long)f_logit.stride(0),
                        fb.data_ptr<float>(), lo.data_ptr<float>(), H * D);
     HIP_CHECK_LAST();
-    launch_scan<false, T>(out.data_ptr<float>(), qa.data_ptr<float>(), (const float*)nullptr, f.data_ptr<float>(),
+    launch_scan<SCAN_TIED, T>(out.data_ptr<float>(), qa.data_ptr<float>(), (const float*)nullptr, f.data_ptr<float>(),
                           (const float*)nullptr, ptr<T>(v), (long)v.stride(0), state.data_ptr<float>(),
                           (long)state.stride(0), cu.data_ptr<int>(), start.data_ptr<int>(), slots.data_ptr<int>(), B, H,
                           1, D, Dv);
+  });
+  return out;
+}
+
+at::Tensor ssd_recurrence(at::Tensor x, at::Tensor Bm, at::Tensor Cm, at::Tensor dt_raw, at::Tensor A_log,
+                          at::Tensor dt_bias, at::Tensor D_skip, at::Tensor state, at::Tensor cu, at::Tensor start,
+                          at::Tensor slots) {
+  check_act(x, "x"); check_act(dt_raw, "dt_raw");
+  TORCH_CHECK(x.dim() == 3 && x.stride(2) == 1 && x.stride(1) == x.size(2), "x must be [N, H, Dv] with dense rows");
+  const long N = x.size(0);
+  const int H = (int)x.size(1), Dv = (int)x.size(2);
+  // B and C feed the recurrence unrounded: float32 rows [N, G, D], dense inside a row, one token stride for both
+  TORCH_CHECK(Bm.is_cuda() && is_f32(Bm) && Cm.is_cuda() && is_f32(Cm) && Bm.dim() == 3 && Bm.sizes() == Cm.sizes() &&
+              Bm.size(0) == N, "B and C must be float32 [N, G, D]");
+  const int G = (int)Bm.size(1), D = (int)Bm.size(2);
+  TORCH_CHECK(Bm.stride(2) == 1 && Cm.stride(2) == 1 && Bm.stride(1) == D && Cm.stride(1) == D &&
+              Bm.stride(0) == Cm.stride(0), "B and C rows must be dense and share a token stride");
+  TORCH_CHECK(G > 0 && H % G == 0, "heads must split evenly into the groups");
+  TORCH_CHECK(dt_raw.dim() == 2 && dt_raw.size(0) == N && dt_raw.size(1) == H && dt_raw.stride(1) == 1);
+  check_state(state, H, D, Dv);
+  check_i32(cu, "cu"); check_i32(start, "start"); check_i32(slots, "slots");
+  const int B = (int)start.numel();
+  at::Tensor Af = f32c(A_log), bf = f32c(dt_bias), Df = f32c(D_skip);
+  TORCH_CHECK(Af.numel() == H && bf.numel() == H && Df.numel() == H && Af.is_cuda() && bf.is_cuda() && Df.is_cuda());
+  auto fo = x.options().dtype(at::kFloat);
+  at::Tensor out = at::empty({N, H, Dv}, fo);
+  if (N == 0) return out;
+  at::Tensor scal = at::empty({N, H, 2}, fo);
+  SERVING_DISPATCH_ACT(dt_raw, TL, {
+    hipLaunchKernelGGL(ssd_prepare_kernel<TL>, dim3((unsigned)((N * H + 255) / 256)), dim3(256), 0, stream(),
+                       scal.data_ptr<float>(), ptr<TL>(dt_raw), (long)dt_raw.stride(0), Af.data_ptr<float>(),
+                       bf.data_ptr<float>(), N, H);
+  });
+  HIP_CHECK_LAST();
+  const int vec_ok = (Bm.stride(0) % 4 == 0 && reinterpret_cast<uintptr_t>(Bm.data_ptr()) % 16 == 0 &&
+                      reinterpret_cast<uintptr_t>(Cm.data_ptr()) % 16 == 0) ? 1 : 0;
+  SERVING_DISPATCH_ACT(x, T, {
+    launch_scan<SCAN_SSD, T>(out.data_ptr<float>(), Cm.data_ptr<float>(), Bm.data_ptr<float>(), (const float*)nullptr,
+                             scal.data_ptr<float>(), ptr<T>(x), (long)x.stride(0), state.data_ptr<float>(),
+                             (long)state.stride(0), cu.data_ptr<int>(), start.data_ptr<int>(), slots.data_ptr<int>(),
+                             B, H, H / G, D, Dv, (long)Bm.stride(0), vec_ok, Df.data_ptr<float>());
   });
   return out;
 }

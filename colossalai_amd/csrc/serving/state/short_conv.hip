@@ -1,4 +1,4 @@
-// Short causal depthwise convolution over a ragged batch, with the last
+// Short causal depthwise convolution (optional bias) over a ragged batch, with the last
 // K-1 inputs of every sequence carried in a state slot.
 //
 // Two launches: the outputs (read the slot's tail, write nothing to it), then
@@ -18,14 +18,14 @@ template <typename T, typename TO>
 __global__ __launch_bounds__(256) void short_conv_kernel(
     TO* __restrict__ y, const T* __restrict__ x, long xs, const float* __restrict__ taps, const float* __restrict__ tail,
     long ts, const int* __restrict__ cu, const int* __restrict__ start, const int* __restrict__ slots,
-    const int* __restrict__ tok_seq, int C, int K, int silu) {
+    const int* __restrict__ tok_seq, int C, int K, int silu, const float* __restrict__ bias) {
   const int n = blockIdx.x;
   const int b = tok_seq[n];
   const int i = n - cu[b];  // index inside the portion
   const bool fresh = start[b] == 0;
   const float* tl = tail + (long)slots[b] * ts;
   for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < C; c += gridDim.y * blockDim.x) {
-    float acc = 0.0f;
+    float acc = bias != nullptr ? bias[c] : 0.0f;
     for (int d = 0; d < K; ++d) {
       float v;
       if (d <= i) v = ldf(x + (long)(n - d) * xs + c);
@@ -63,7 +63,8 @@ __global__ __launch_bounds__(256) void short_conv_tail_kernel(
 }
 
 at::Tensor short_conv(at::Tensor x, at::Tensor taps, c10::optional<at::Tensor> tail, at::Tensor cu, at::Tensor start,
-                      at::Tensor slots, at::Tensor tok_seq, bool silu, at::ScalarType out_dtype) {
+                      at::Tensor slots, at::Tensor tok_seq, bool silu, at::ScalarType out_dtype,
+                      c10::optional<at::Tensor> bias) {
   check_act(x, "x");
   TORCH_CHECK(x.dim() == 2 && x.stride(1) == 1, "x must be [N, C] with unit inner stride");
   const long N = x.size(0);
@@ -71,7 +72,13 @@ at::Tensor short_conv(at::Tensor x, at::Tensor taps, c10::optional<at::Tensor> t
   TORCH_CHECK(taps.dim() == 2 && taps.size(0) == C && K >= 1 && K <= MAX_TAPS, "taps must be [C, K], K <= 16");
   check_i32(cu, "cu"); check_i32(start, "start"); check_i32(slots, "slots"); check_i32(tok_seq, "tok_seq");
   TORCH_CHECK(tok_seq.numel() == N);
-  at::Tensor tp = f32c(taps);
+  at::Tensor tp = f32c(taps), bs;
+  const float* bp = nullptr;
+  if (bias.has_value()) {
+    bs = f32c(*bias);
+    TORCH_CHECK(bs.numel() == C && bs.is_cuda(), "bias must be [C]");
+    bp = bs.data_ptr<float>();
+  }
   at::Tensor y = at::empty({N, C}, x.options().dtype(out_dtype));
   if (N == 0) return y;
   const float* tlp = nullptr;
@@ -91,7 +98,7 @@ at::Tensor short_conv(at::Tensor x, at::Tensor taps, c10::optional<at::Tensor> t
     SERVING_DISPATCH_ACT(y, TO, {
       hipLaunchKernelGGL((short_conv_kernel<T, TO>), dim3((unsigned)N, gy), dim3(256), 0, stream(), ptr<TO>(y), ptr<T>(x),
                          (long)x.stride(0), tp.data_ptr<float>(), tlp, ts, cu.data_ptr<int>(), start.data_ptr<int>(),
-                         slots.data_ptr<int>(), tok_seq.data_ptr<int>(), C, K, (int)silu);
+                         slots.data_ptr<int>(), tok_seq.data_ptr<int>(), C, K, (int)silu, bp);
     });
     if (K > 1)
       hipLaunchKernelGGL(short_conv_tail_kernel<T>, dim3((unsigned)B, gy), dim3(256), 0, stream(), ptr<T>(x),
