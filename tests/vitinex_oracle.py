@@ -54,6 +54,21 @@ def rotate_pairs(x, positions, base, dims):
     return out
 
 
+def latent_attention_core(q, q_rot, lat, k_rot, w_uk, w_uv, scale, q_pos, k_pos):
+    """q [T, H, D] plain and q_rot [T, H, R] rotated query parts; lat [S, rank] normed latents and k_rot [S, R] the
+    rotated key part all heads share; w_uk [H * D, rank], w_uv [H * Dv, rank]. Head h's key is its slice of
+    ``w_uk lat`` next to ``k_rot``, its value its slice of ``w_uv lat``; query i sees the keys j with
+    k_pos[j] <= q_pos[i]. Returns [T, H, Dv]."""
+    T, H, D = q.shape
+    S = lat.shape[0]
+    k_plain = lin(lat, w_uk).view(S, H, D)
+    v = lin(lat, w_uv).view(S, H, -1)
+    score = (torch.einsum("thd,shd->hts", q, k_plain) + torch.einsum("thr,sr->hts", q_rot, k_rot)) * scale
+    seen = q_pos.view(-1, 1) >= k_pos.view(1, -1)
+    score = score.masked_fill(~seen, float("-inf"))
+    return torch.einsum("hts,shv->thv", torch.softmax(score, -1), v)
+
+
 def latent_attention(h, P, pre, c, eps, positions=None):
     """Queries through a normed latent; keys and values up-projected from a normed latent; one rotated key part
     shared by all heads; causal softmax; per-head sigmoid output gate."""
@@ -66,12 +81,7 @@ def latent_attention(h, P, pre, c, eps, positions=None):
     lat = rms_unit(dkv[:, :rank], eps) * P[pre + "dkv.norm"].to(F64)
     k_rot = rotate_pairs(dkv[:, rank:].clone(), pos, c["rot"]["base"], c["rot"]["dims"])     # [T, R]
     q_rot = rotate_pairs(q[..., D:].clone(), pos, c["rot"]["base"], c["rot"]["dims"])        # [T, H, R]
-    k_plain = lin(lat, P[pre + "uk"]).view(T, H, D)
-    v = lin(lat, P[pre + "uv"]).view(T, H, Dv)
-    score = (torch.einsum("thd,shd->hts", q[..., :D], k_plain) + torch.einsum("thr,sr->hts", q_rot, k_rot)) * c["scale"]
-    seen = pos.view(-1, 1) >= pos.view(1, -1)
-    score = score.masked_fill(~seen, float("-inf"))
-    o = torch.einsum("hts,shv->thv", torch.softmax(score, -1), v)
+    o = latent_attention_core(q[..., :D], q_rot, lat, k_rot, P[pre + "uk"], P[pre + "uv"], c["scale"], pos, pos)
     o = o * torch.sigmoid(lin(h, P[pre + "g"]))[:, :, None]
     return lin(o.reshape(T, H * Dv), P[pre + "o"])
 
@@ -88,18 +98,19 @@ def causal_conv(x, taps, bias, history=None):
 
 
 def ssd_scan(x, B, C, dt, A_log, D_skip, groups, S0=None):
-    """x [T, H, V], B/C [T, G, N], dt [T, H] (after softplus). S_t = exp(-exp(A_log) dt) S + dt B x^T; y = S^T C + D x."""
+    """x [T, H, V], B/C [T, G, N], dt [T, H] (after softplus). Per head h (group h // (H / G)):
+    S_t = exp(-exp(A_log_h) dt) S_(t-1) + dt B_t x_t^T (S is N x V); y_t = S_t^T C_t + D_h x_t. Token by token."""
     T, H, V = x.shape
     N = B.shape[2]
     S = torch.zeros(H, N, V, dtype=F64) if S0 is None else S0.clone()
     y = torch.zeros(T, H, V, dtype=F64)
     per = H // groups
+    head_group = torch.arange(H) // per
     for t in range(T):
-        for hd in range(H):
-            g = hd // per
-            decay = math.exp(-math.exp(float(A_log[hd])) * float(dt[t, hd]))
-            S[hd] = decay * S[hd] + float(dt[t, hd]) * torch.outer(B[t, g], x[t, hd])
-            y[t, hd] = S[hd].T @ C[t, g] + float(D_skip[hd]) * x[t, hd]
+        Bt, Ct = B[t][head_group], C[t][head_group]                      # [H, N]
+        decay = torch.exp(-torch.exp(A_log.to(F64)) * dt[t])             # [H]
+        S = decay[:, None, None] * S + dt[t][:, None, None] * Bt[:, :, None] * x[t][:, None, :]
+        y[t] = torch.einsum("hnv,hn->hv", S, Ct) + D_skip.to(F64)[:, None] * x[t]
     return y, S
 
 
