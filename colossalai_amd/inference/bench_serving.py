@@ -1,9 +1,11 @@
 """Serving throughput of the ragged-step models next to a Llama of equal width,
 depth and per-token work, all through ``ContinuousBatchEngine``: prefill tokens/s
 of one long prompt and decode tokens/s of a batch of running sequences. Random
-weights, synthetic tokens. Two comparisons: the Kipirax hybrid (paged window
-attention + recurrent state) and Mubutar (sink-softmax attention with shared
-keys, routed experts).
+weights, synthetic tokens. Three comparisons: the Kipirax hybrid (paged window
+attention + recurrent state), Mubutar (sink-softmax attention with shared
+keys, routed experts) and Vitinex (latent attention + state-space layers in a
+looped block, routed experts), the last also next to Mubutar, whose kernels are
+the closest.
 """
 
 import json
@@ -13,11 +15,11 @@ from typing import Dict, List
 import torch
 
 from ..models import (KipiraxConfig, KipiraxForCausalLM, LlamaConfig, LlamaForCausalLM, MubutarConfig,
-                      MubutarForCausalLM)
+                      MubutarForCausalLM, VitinexConfig, VitinexForCausalLM)
 from .config import InferenceConfig
 from .paged_engine import ContinuousBatchEngine
 
-__all__ = ["SIZES", "hybrid_config", "llama_config", "moe_config", "run_serving_comparison"]
+__all__ = ["SIZES", "hybrid_config", "llama_config", "moe_config", "latent_config", "run_serving_comparison"]
 
 # width, layers, heads, kv_heads, head size, vocab
 SIZES = {
@@ -65,6 +67,29 @@ def moe_config(s: dict, experts: int = 32, top: int = 6) -> MubutarConfig:
                          logit_scale=1.0)
 
 
+def latent_config(s: dict, experts: int = 32, top: int = 6) -> VitinexConfig:
+    """As many layer runs as the size has layers: latent attention and state-space layers in turn, the first two
+    looped twice. Per head 64 plain + 64 rotated key channels and 128 value channels (Llama's head size), a latent
+    of a quarter of Llama's keys + values per token; the state-space layers are twice the width inside, heads of
+    64 channels, a state of 128 per head in 8 groups. Even layers carry Llama's dense feed-forward, odd ones
+    Mubutar's expert sizes."""
+    W, H, D = s["width"], s["heads"], s["dim"]
+    inter = _inter(W)
+    ff = W // 2
+    shared = (3 * inter // 2 - top * ff + 127) // 128 * 128
+    lat = dict(dim=D // 2, rot_dim=D // 2, vdim=D, heads=H, kv_rank=2 * D, q_rank=3 * W // 8,
+               rot=dict(base=10000.0, dims=D // 2), scale=D ** -0.5)
+    ssm = dict(conv=4, groups=8, heads=2 * W // 64, norm_groups=8, state=128, vdim=64)
+    layers = []
+    for i in range(s["layers"] - 2):
+        mixer = ("latent_attention", lat) if i % 2 == 0 else ("mamba2", ssm)
+        mlp = dict(kind="dense", ff=inter) if i % 2 == 0 else dict(
+            kind="moe", expert=dict(ff=ff), shared=dict(ff=shared), router=dict(experts=experts, top=top))
+        layers.append(dict(type=mixer[0], mixer=mixer[1], mlp=mlp))
+    return VitinexConfig(vocab=s["vocab"], width=W, layers=layers, norm_eps=1e-6, residual_mult=0.5,
+                         loop=dict(start=0, stop=2, times=2))
+
+
 def llama_config(s: dict, max_positions: int) -> LlamaConfig:
     # gate/up/down of 8/3 W carry the parameters of the hybrid's up/down of 4 W
     inter = _inter(s["width"])
@@ -107,6 +132,23 @@ def _moe_numbers(s: dict, prompt: int, batch: int, context: int, steps: int) -> 
         layer.mix.in_proj.bias.data = layer.mix.in_proj.bias.data.to(torch.bfloat16)
     out = _ragged_numbers(model, cfg.vocab, prompt, batch, context, steps)
     return out
+
+
+def _latent_numbers(s: dict, prompt: int, batch: int, context: int, steps: int) -> Dict[str, float]:
+    cfg = latent_config(s)
+    model = _random(VitinexForCausalLM(cfg), torch.bfloat16)
+    with torch.no_grad():
+        model.loop_in.data = model.loop_in.data.float()     # the loop's mix and the routers stay float32
+        model.loop_step.data = model.loop_step.data.float()
+        for layer in model.layers:
+            if hasattr(layer.mlp, "router"):
+                layer.mlp.router.data = layer.mlp.router.data.float()
+            if hasattr(layer.mlp, "in_proj"):
+                layer.mlp.in_proj.bias.data = layer.mlp.in_proj.bias.data.to(torch.bfloat16)
+                layer.mlp.down.bias.data = layer.mlp.down.bias.data.to(torch.bfloat16)
+            if layer.kind == "mamba2":
+                layer.mix.conv.data = layer.mix.conv.data.float().normal_(0, 0.3)
+    return _ragged_numbers(model, cfg.vocab, prompt, batch, context, steps)
 
 
 def _ragged_numbers(model, vocab: int, prompt: int, batch: int, context: int, steps: int) -> Dict[str, float]:
@@ -164,12 +206,15 @@ def _llama_numbers(s: dict, prompt: int, batch: int, context: int, steps: int) -
 
 def run_serving_comparison(sizes: List[str], prompt: int = 4096, batch: int = 16, context: int = 1024,
                            steps: int = 32, kind: str = "hybrid") -> dict:
-    """``kind``: "hybrid" (Kipirax) or "moe" (Mubutar), each next to Llama."""
-    ours = {"hybrid": _hybrid_numbers, "moe": _moe_numbers}[kind]
+    """``kind``: "hybrid" (Kipirax), "moe" (Mubutar) or "latent" (Vitinex), each next to Llama; "latent" also
+    next to Mubutar."""
+    ours = {"hybrid": _hybrid_numbers, "moe": _moe_numbers, "latent": _latent_numbers}[kind]
     out = {}
     for name in sizes:
         s = SIZES[name]
-        out[name] = {kind: ours(s, prompt, batch, context, steps),
-                     "llama": _llama_numbers(s, prompt, batch, context, steps),
-                     "shape": dict(s, prompt=prompt, batch=batch, context=context)}
+        out[name] = {kind: ours(s, prompt, batch, context, steps)}
+        if kind == "latent":
+            out[name]["moe"] = _moe_numbers(s, prompt, batch, context, steps)
+        out[name]["llama"] = _llama_numbers(s, prompt, batch, context, steps)
+        out[name]["shape"] = dict(s, prompt=prompt, batch=batch, context=context)
     return out

@@ -31,6 +31,7 @@ class RaggedBatch:
     start_host: List[int]
     slots_host: List[int]
     page_size: int = 0
+    _dense: Optional[tuple] = None  # memo of dense_context()
 
     @property
     def num_seqs(self) -> int:
@@ -56,6 +57,34 @@ class RaggedBatch:
     def max_total(self) -> int:
         """Longest sequence after this step (cached + new tokens)."""
         return max(self.start_host[i] + self.cu_host[i + 1] - self.cu_host[i] for i in range(self.num_seqs))
+
+    def dense_context(self):
+        """For ops that lay the whole context of the step's sequences (cached and new tokens) out densely, each
+        sequence padded to whole pages: ``(rows, tables, total)`` with ``rows`` [total] the pool row of every place
+        of that layout (a padding place repeats the sequence's last row) and ``tables`` [B, max_pages] int32 the page
+        table of the dense layout itself (consecutive pages, sequence after sequence). Built on the device from
+        the step's own index vectors, once per step."""
+        if self._dense is None:
+            ps, dev = self.page_size, self.cu.device
+            shift = ps.bit_length() - 1
+            lens = [self.start_host[i] + self.cu_host[i + 1] - self.cu_host[i] for i in range(self.num_seqs)]
+            pages = [(n + ps - 1) // ps for n in lens]
+            first, total_pages = [], 0
+            for n in pages:
+                first.append(total_pages)
+                total_pages += n
+            width = max(pages)
+            host = torch.tensor([first, pages, lens], dtype=torch.int32).to(dev)   # one copy
+            first_d, pages_d, lens_d = host[0].long(), host[1].long(), host[2].long()
+            total = total_pages * ps
+            seq = torch.repeat_interleave(torch.arange(self.num_seqs, device=dev), pages_d * ps, output_size=total)
+            pos = torch.arange(total, device=dev) - first_d[seq] * ps
+            pos = torch.minimum(pos, lens_d[seq] - 1)
+            rows = (self.block_tables[seq, pos >> shift].long() << shift) + (pos & (ps - 1))
+            cols = torch.arange(width, device=dev)
+            tables = torch.where(cols[None, :] < pages_d[:, None], first_d[:, None] + cols[None, :], 0).int()
+            self._dense = (rows, tables.contiguous(), total)
+        return self._dense
 
     @classmethod
     def build(cls, new_counts: Sequence[int], starts: Sequence[int], slots: Sequence[int], device,
