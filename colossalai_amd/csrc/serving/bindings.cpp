@@ -20,7 +20,7 @@ at::Tensor merge_rms_norm(at::Tensor a, at::Tensor wa, at::Tensor b, at::Tensor 
 at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at::Tensor block_tables, at::Tensor cu,
                            at::Tensor start, at::Tensor tok_seq, at::Tensor positions, double scale, int64_t window,
                            int64_t keep_first, c10::optional<at::Tensor> slopes, c10::optional<at::Tensor> gate,
-                           int64_t num_tiles, double softcap, bool sink);
+                           int64_t num_tiles, double softcap, bool sink, int64_t num_tiles128);
 at::Tensor silu_mul(at::Tensor packed);
 c10::optional<at::Tensor> add_rms_norm(at::Tensor residual, at::Tensor a, c10::optional<at::Tensor> b,
                                        c10::optional<at::Tensor> weight, double eps, at::ScalarType out_dtype);

@@ -264,7 +264,12 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     bf16s* __restrict__ out, const bf16s* __restrict__ q, long q_stride, const bf16s* __restrict__ kpool,
     const bf16s* __restrict__ vpool, const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ cu,
     const int* __restrict__ start, const float* __restrict__ slopes, const bf16s* __restrict__ gate, long gate_stride,
-    int H, int G, int Dr, int Dvr, int page_shift, float scale, int window, int keep_first, float softcap, int sink) {
+    int H, int G, int Dr, int Dvr, int page_shift, float scale, int window, int keep_first, float softcap, int sink,
+    int qsplit) {
+  // qsplit (kv heads with a single query head each): the four waves of a block are four consecutive 32-token tiles
+  // of that head instead of four heads, so a block covers 128 tokens, the grid's x axis counts 128-token tiles, and
+  // the staged key/value tiles are still shared by all computing waves. The block stages the key range of all its
+  // tokens; a wave skips the tiles that lie wholly after its own tokens.
   constexpr int D = DS * 16, Dv = VT * 32;
   bf16x8_v zero8;
 #pragma unroll
@@ -279,29 +284,32 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   const int tid = threadIdx.x;
   const int wid = tid >> 6, lane = tid & 63;
   const int rep = H / G, g = blockIdx.y;
-  const int hl = blockIdx.z * (nthreads >> 6) + wid;  // head inside the group
-  const bool head_ok = hl < rep;
-  const int h = g * rep + (head_ok ? hl : 0);
+  const int hl = qsplit ? 0 : blockIdx.z * (nthreads >> 6) + wid;  // head inside the group
+  const int h = g * rep + (hl < rep ? hl : 0);
+  const int bshift = qsplit ? 7 : 5;                  // log2 of the tokens a block covers
   // Under a causal mask a late tile of a long prompt has many more key tiles than an early one. Rows of the grid
   // (kv head, pass) walk the tiles alternately from the back and from the front, switching with every 256 blocks of
   // dispatch order, so that blocks which come to share a CU tend to pair a long tile with a short one and the
   // longest tiles start first.
   const bool from_back = ((gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z)) >> 8 & 1) == 0;
   int tile = from_back ? gridDim.x - 1 - blockIdx.x : blockIdx.x, b = 0;
-  for (;; ++b) {  // the grid holds exactly sum_b ceil(count_b / 32) tiles
-    const int nt = (cu[b + 1] - cu[b] + 31) >> 5;
+  for (;; ++b) {  // the grid holds exactly sum_b ceil(count_b / tokens per block) tiles
+    const int nt = (cu[b + 1] - cu[b] + (1 << bshift) - 1) >> bshift;
     if (tile < nt) break;
     tile -= nt;
   }
   const int cnt = cu[b + 1] - cu[b];
   const int col = lane & 31, hf = lane >> 5;
-  const int t_off = tile * 32;
+  const int bt_off = tile << bshift;                          // first token of the block
+  const int t_off = bt_off + (qsplit ? wid * 32 : 0);         // first token of this wave
+  const bool head_ok = qsplit ? t_off < cnt : hl < rep;       // this wave computes
   const bool tok_ok = t_off + col < cnt;
   const int my_i = tok_ok ? t_off + col : cnt - 1;
   const long n = cu[b] + my_i;
   const int s0 = start[b];
   const int pos = s0 + my_i;
-  const int p0 = s0 + t_off, p1 = s0 + min(t_off + 31, cnt - 1);
+  const int p0 = s0 + t_off, p1 = s0 + min(t_off + 31, cnt - 1);              // this wave's positions
+  const int bp0 = s0 + bt_off, bp1 = s0 + min(bt_off + (1 << bshift) - 1, cnt - 1);  // the block's
   const int* bt = block_tables + (long)b * bt_stride;
   const int page_mask = (1 << page_shift) - 1;
   const float slope = slopes != nullptr ? slopes[h] : 0.0f;
@@ -311,11 +319,11 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   for (int s = 0; s < DS; ++s)
     qf[s] = 16 * s + hf * 8 < Dr ? ld_g16b(q + n * q_stride + (long)h * Dr + 16 * s + hf * 8) : zero8;
 
-  const int lo_min = window > 0 ? max(0, p0 - window + 1) : 0;
+  const int lo_min = window > 0 ? max(0, bp0 - window + 1) : 0;   // the staged key range is the block's
   const int wstart = lo_min & ~31;
   const int n_sink = window > 0 ? min(keep_first, wstart) : 0;  // kept keys below the window's first tile
   const int sink_tiles = (n_sink + 31) >> 5;
-  const int tiles_n = sink_tiles + ((p1 - wstart) >> 5) + 1;
+  const int tiles_n = sink_tiles + ((bp1 - wstart) >> 5) + 1;
 
   // staging: key chunk c = key c / (row chunks), 8 elements starting at 8 * (c % row chunks), stored as a row;
   // value chunk c = key c % 32, 8 channels starting at 8 * (c / 32): the values are stored transposed, two bytes at
@@ -326,7 +334,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   bf16x8_v rk[TP][KR], rv[TP][VR];
   auto tile_base = [&](int it) { return it < sink_tiles ? it * 32 : wstart + (it - sink_tiles) * 32; };
   auto pool_row = [&](int j) {
-    const int jc = min(j, p1);  // keys past the sequence's end are masked; read a row that exists
+    const int jc = min(j, bp1);  // keys past the sequence's end are masked; read a row that exists
     return ((long)bt[jc >> page_shift] << page_shift) + (jc & page_mask);
   };
   // The page-table lookups of a tile run one tile ahead of its key/value loads (two ahead of its use), so that a
@@ -441,6 +449,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
       if (!head_ok || it >= tiles_n) continue;
       const bool sink = it < sink_tiles;
       const int kbase = tile_base(it);
+      if (!sink && kbase > p1) continue;  // (query split) a tile wholly after this wave's tokens
       const int klimit = sink ? n_sink : p1 + 1;  // keys of this tile at or above it are not this tile's to count
       const bf16s* ks = tiles + (buf * TP + u) * (KT + VTT);
       const bf16s* vt = ks + KT;
@@ -532,7 +541,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
 at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at::Tensor block_tables, at::Tensor cu,
                            at::Tensor start, at::Tensor tok_seq, at::Tensor positions, double scale, int64_t window,
                            int64_t keep_first, c10::optional<at::Tensor> slopes, c10::optional<at::Tensor> gate,
-                           int64_t num_tiles, double softcap, bool sink) {
+                           int64_t num_tiles, double softcap, bool sink, int64_t num_tiles128) {
   check_act(q, "q");
   TORCH_CHECK(softcap >= 0.0, "softcap must not be negative (0 = none)");
   TORCH_CHECK(q.dim() == 3 && q.stride(2) == 1 && q.stride(1) == q.size(2), "q must be [N, H, D] with dense rows");
@@ -576,7 +585,9 @@ at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at:
   const bool mfma_shape = D % 8 == 0 && Dv % 8 == 0 && D <= 128 && Dv <= 128;
   if (num_tiles > 0 && is_bf16(q) && aligned && mfma_shape && vpool.is_contiguous()) {
     const int rep = H / G, nw = 4;
-    const dim3 grid((unsigned)num_tiles, (unsigned)G, (unsigned)((rep + nw - 1) / nw));
+    // one query head per kv head: the waves of a block take four consecutive token tiles instead of four heads
+    const int qsplit = (rep == 1 && num_tiles128 > 0) ? 1 : 0;
+    const dim3 grid((unsigned)(qsplit ? num_tiles128 : num_tiles), (unsigned)G, (unsigned)((rep + nw - 1) / nw));
     const int ds = D <= 32 ? 2 : D <= 48 ? 3 : D <= 64 ? 4 : D <= 96 ? 6 : 8, vt = (Dv + 31) / 32;
     const size_t msmem = (size_t)2 * MFMA_TILES_PER_STEP * (32 * (ds * 16 + 8) + vt * 32 * 40) * sizeof(bf16s);
 #define MFMA_CASE(DS_, VT_)                                                                                        \
@@ -588,7 +599,8 @@ at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at:
                        (long)q.stride(0), ptr<bf16s>(kpool), ptr<bf16s>(vpool), block_tables.data_ptr<int>(),      \
                        (int)block_tables.stride(0), cu.data_ptr<int>(), start.data_ptr<int>(), slp,                \
                        gate.has_value() ? ptr<bf16s>(*gate) : (const bf16s*)nullptr, gstride, H, G, D, Dv,         \
-                       page_shift, (float)scale, (int)window, (int)keep_first, (float)softcap, sink ? 1 : 0);      \
+                       page_shift, (float)scale, (int)window, (int)keep_first, (float)softcap, sink ? 1 : 0,       \
+                       qsplit);                                                                                    \
   } while (0)
 #define MFMA_ROW(DS_)                     \
   do {                                    \

@@ -300,10 +300,15 @@ __global__ __launch_bounds__(256) void matrix_state_scan_kernel(
 template <int MODE, typename TV>
 static void launch_scan(float* out, const float* q, const float* k, const float* gate, const float* beta, const TV* v,
                         long vs, float* state, long ss, const int* cu, const int* start, const int* slots, int B,
-                        int H, int rep, int D, int Dv, long qk_ts = 0, int vec_ok = 1, const float* skip = nullptr) {
+                        int H, int rep, int D, int Dv, long qk_ts = 0, int vec_ok = 1, const float* skip = nullptr,
+                        bool short_step = false) {
   constexpr bool DELTA = MODE == SCAN_DELTA;
   TORCH_CHECK(D <= 256, "key size above 256 is not supported by the recurrence kernel");
-  const int dpl = D > 128 ? 16 : 8;
+  // A step of single tokens (decoding) is all state traffic: a lane then holds 32 rows of its channel, so that few
+  // lanes share a channel, a wave's loads of one state row cover 16 to 64 neighbouring channels and a block 64 to
+  // 256 (whole cache lines), instead of 4 channels per wave when 16 lanes split a channel of 128 rows.
+  const bool wide = MODE == SCAN_SSD && short_step;
+  const int dpl = wide ? 32 : D > 128 ? 16 : 8;
   int P = 1;
   while (P * dpl < D) P <<= 1;
   const int cpb = 4 * 64 / P /* times NC of the kernel */, Dp = P * dpl, ct = Dp > 128 ? 8 : 16, nops = DELTA ? 3 : 2;
@@ -312,6 +317,16 @@ static void launch_scan(float* out, const float* q, const float* k, const float*
 #define SCAN_CASE(PP, DD)                                                                                          \
   hipLaunchKernelGGL((matrix_state_scan_kernel<PP, DD, MODE, TV>), grid, dim3(256), smem, stream(), out, q, k,    \
                      gate, beta, v, vs, state, ss, cu, start, slots, H, rep, D, Dv, qk_ts, vec_ok, skip)
+  if constexpr (MODE == SCAN_SSD) {
+    if (wide) {
+      if (P == 1) SCAN_CASE(1, 32);
+      else if (P == 2) SCAN_CASE(2, 32);
+      else if (P == 4) SCAN_CASE(4, 32);
+      else SCAN_CASE(8, 32);
+      HIP_CHECK_LAST();
+      return;
+    }
+  }
   if (dpl == 16) SCAN_CASE(16, 16);
   else if (P == 1) SCAN_CASE(1, 8);
   else if (P == 2) SCAN_CASE(2, 8);
@@ -437,7 +452,7 @@ at::Tensor ssd_recurrence(at::Tensor x, at::Tensor Bm, at::Tensor Cm, at::Tensor
     launch_scan<SCAN_SSD, T>(out.data_ptr<float>(), Cm.data_ptr<float>(), Bm.data_ptr<float>(), (const float*)nullptr,
                              scal.data_ptr<float>(), ptr<T>(x), (long)x.stride(0), state.data_ptr<float>(),
                              (long)state.stride(0), cu.data_ptr<int>(), start.data_ptr<int>(), slots.data_ptr<int>(),
-                             B, H, H / G, D, Dv, (long)Bm.stride(0), vec_ok, Df.data_ptr<float>());
+                             B, H, H / G, D, Dv, (long)Bm.stride(0), vec_ok, Df.data_ptr<float>(), N <= 2L * B);
   });
   return out;
 }

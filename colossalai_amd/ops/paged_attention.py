@@ -89,5 +89,6 @@ def paged_attention(q, kpool, vpool, batch: RaggedBatch, scale: float, window: i
     if use_hip(q):
         return serving_kernels().paged_attention(q, kpool, vpool, batch.block_tables, batch.cu, batch.start,
                                                  batch.tok_seq, batch.positions, scale, window, keep_first,
-                                                 slopes, gate, batch.num_tiles32, float(softcap), bool(sink))
+                                                 slopes, gate, batch.num_tiles32, float(softcap), bool(sink),
+                                                 batch.num_tiles128)
     return paged_attention_ref(q, kpool, vpool, batch, scale, window, keep_first, slopes, gate, softcap, sink)

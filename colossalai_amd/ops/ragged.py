@@ -54,6 +54,14 @@ class RaggedBatch:
         return sum((self.cu_host[i + 1] - self.cu_host[i] + 31) // 32 for i in range(self.num_seqs))
 
     @property
+    def num_tiles128(self) -> int:
+        """128-token tiles of the prompt portions (0 for a pure decode step): the grid of the matrix-core attention
+        kernel when every key head has a single query head."""
+        if self.max_new == 1:
+            return 0
+        return sum((self.cu_host[i + 1] - self.cu_host[i] + 127) // 128 for i in range(self.num_seqs))
+
+    @property
     def max_total(self) -> int:
         """Longest sequence after this step (cached + new tokens)."""
         return max(self.start_host[i] + self.cu_host[i + 1] - self.cu_host[i] for i in range(self.num_seqs))

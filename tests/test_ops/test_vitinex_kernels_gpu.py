@@ -187,3 +187,44 @@ def test_experts_with_gated_base(dtype, N):
                                            "relu_squared", wide.cuda()[:, E])
     ref = routed_experts.routed_expert_ffn_ref(h, up, down, ids, wt, base, "relu_squared", wide[:, E])
     torch.testing.assert_close(out.cpu(), ref, **(dict(rtol=1e-4, atol=1e-4) if dtype == torch.float32 else tol(dtype)))
+
+
+@pytest.mark.parametrize("window,keep", [(0, 0), (70, 5)])
+@pytest.mark.parametrize("D,Dv", [(64, 32), (128, 128), (48, 24)])
+def test_one_query_head_per_key_head_prompt_tiles(window, keep, D, Dv):
+    """Multi-head attention without grouping in bfloat16: the matrix-core kernel's blocks take four token tiles of
+    one head. Portions longer and shorter than a block, from position 0 and continued, next to a decode token."""
+    torch.manual_seed(11)
+    counts, starts, page = [200, 37, 1, 130, 128], [0, 50, 9, 300, 64], 16
+    tables, nxt = [], 0
+    for c, s in zip(counts, starts):
+        need = (c + s + page - 1) // page
+        tables.append(list(range(nxt + need - 1, nxt - 1, -1)))
+        nxt += need
+    gb = RaggedBatch.build(counts, starts, list(range(5)), "cuda", tables, page)
+    cb = RaggedBatch.build(counts, starts, list(range(5)), "cpu", tables, page)
+    H = 3
+    kpool = (torch.randn(nxt, page, H, D) * 0.5).to(torch.bfloat16)
+    vpool = torch.randn(nxt, page, H, Dv).to(torch.bfloat16)
+    q = (torch.randn(gb.num_tokens, H, D) * 0.5).to(torch.bfloat16)
+    gate = torch.randn(gb.num_tokens, H).to(torch.bfloat16)
+    out = paged_attention(q.cuda(), kpool.cuda(), vpool.cuda(), gb, 0.3, window, keep, None, gate.cuda())
+    ref = paged_attention_ref(q, kpool, vpool, cb, 0.3, window, keep, None, gate)
+    torch.testing.assert_close(out.cpu().float(), ref.float(), rtol=2e-2, atol=2e-2)
+
+
+def test_decode_steps_of_the_state_space_scan_match_prompt_steps():
+    """Single-token steps take a launch shape of their own: same results, same state, as one portion."""
+    torch.manual_seed(12)
+    H, G, D, Dv, T = 8, 2, 128, 64, 6
+    x, Bm, Cm = torch.randn(T, H, Dv).cuda(), torch.randn(T, G, D).cuda(), torch.randn(T, G, D).cuda()
+    dt = torch.randn(T, H).cuda()
+    A_log, dt_bias, skip = (torch.randn(H) * 0.3).cuda(), torch.randn(H).cuda(), torch.randn(H).cuda()
+    st1, st2 = torch.randn(3, H, D, Dv).cuda(), None
+    st2 = st1.clone()
+    whole = linear_recurrence.ssd_recurrence(x, Bm, Cm, dt, A_log, dt_bias, skip, st1,
+                                             RaggedBatch.build([T], [5], [1], "cuda"))
+    steps = [linear_recurrence.ssd_recurrence(x[t : t + 1], Bm[t : t + 1], Cm[t : t + 1], dt[t : t + 1], A_log, dt_bias,
+                                              skip, st2, RaggedBatch.build([1], [5 + t], [1], "cuda")) for t in range(T)]
+    torch.testing.assert_close(torch.cat(steps, 0), whole, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(st2, st1, rtol=1e-5, atol=1e-5)
