@@ -40,9 +40,9 @@ DEV_INLINE float reduce8(float v) { return dpp_add<0x141>(dpp_add<0x4E>(dpp_add<
 // Values: lane = a pair of value channels, the block's weights and pool rows come from LDS.
 // RC = query heads per block: 4 shares each key/value read between the most heads; 2 or 1 are
 // chosen when a decode step would otherwise leave most CUs without a block (the re-reads hit L2).
-// V8 (value head sizes 8, 16, ..., 256): a lane takes 8 consecutive value channels of a key with one 16/32-byte
-// load, Dv / 8 lanes cover a key's row and the 64 / (Dv / 8) lane groups take different keys of the block, so a
-// block of 64 keys is read by Dv / 8 load instructions instead of 64; the groups' sums meet in a butterfly of
+// V8 (value head sizes that are multiples of 8 up to 512): a lane takes 8 consecutive value channels of a key with
+// one 16/32-byte load, vl = Dv / 8 rounded up to a power of two lanes cover a key's row and the 64 / vl lane groups
+// take different keys of the block, so a block of 64 keys is read by vl load instructions instead of 64; the groups' sums meet in a butterfly of
 // shuffles after the last block.
 template <typename T, int RC, bool V8>
 __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
@@ -96,10 +96,12 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
 #pragma unroll
     for (int i = 0; i < NA; ++i) acc[r][i] = 0.0f;
   }
-  const int vl = Dv >> 3;                     // V8: lanes per key row (a power of two) ...
+  int vl = 1;                                 // V8: lanes per key row: the power of two that holds Dv / 8 ...
+  while (vl * 8 < Dv) vl <<= 1;               // (lanes of a row beyond Dv / 8 idle when Dv / 8 is no power of two)
   const int vks = V8 ? 64 / vl : 1;           // ... keys per load instruction ...
   const int vsub = V8 ? lane / vl : 0;        // ... this lane's key group ...
   const int vch = V8 ? (lane % vl) * 8 : 0;   // ... and its first value channel
+  const bool vlive = vch < Dv;
 
   for (int base = wid * 64; base < total; base += 64 * nw) {
     const int cnt = min(64, total - base);
@@ -171,7 +173,12 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
 #pragma unroll 4
       for (int jj = vsub; jj < cnt; jj += vks) {
         float v[8];
-        load8(vpool + (long)prow[jj] * vrow + (long)g * vhead + vch, v);
+        if (vlive) {
+          load8(vpool + (long)prow[jj] * vrow + (long)g * vhead + vch, v);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[e] = 0.0f;
+        }
 #pragma unroll
         for (int r = 0; r < RC; ++r) {
           const float w = pw[r * 64 + jj];
@@ -213,7 +220,7 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
       for (int e = 0; e < 8; ++e) {
         float v = acc[r][e];
         for (int off = vl; off < 64; off <<= 1) v += __shfl_xor(v, off);  // the key groups' sums of this channel
-        if (vsub == 0) mine[r * PS + 2 + vch + e] = v;
+        if (vsub == 0 && vlive) mine[r * PS + 2 + vch + e] = v;
       }
     } else {
       const int dva = 2 * lane, dvb = 128 + 2 * lane;
@@ -633,10 +640,10 @@ at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at:
   TORCH_CHECK(smem <= 64 * 1024, "head sizes too large for the scalar attention kernel");
   const int kvec = D % 8 == 0 ? 1 : 0;   // 16-byte (bfloat16) / 32-byte (float32) aligned key slices
   const int vvec_even = Dv % 2 == 0 ? 1 : 0;
-  // value rows of 8, 16, ..., 256 channels whose loads are aligned take the 8-channels-per-lane value phase
-  const bool v8 = Dv >= 8 && (Dv & (Dv - 1)) == 0 && reinterpret_cast<uintptr_t>(vpool.data_ptr()) % 32 == 0 &&
+  // value rows of a multiple of 8 channels whose loads are aligned take the 8-channels-per-lane value phase
+  const bool v8 = Dv >= 8 && Dv % 8 == 0 && reinterpret_cast<uintptr_t>(vpool.data_ptr()) % 32 == 0 &&
                   vrow % 8 == 0 && vhead % 8 == 0;
-  TORCH_CHECK(v8 || Dv <= 256, "value rows above 256 channels must be a power of two and aligned");
+  TORCH_CHECK(v8 || Dv <= 256, "value rows above 256 channels must be a multiple of 8 channels and aligned");
   const int vvec_ok = (vrow % 2 == 0 && vhead % 2 == 0) ? 1 : 0;
 #define SCALAR_CASE(RC_)                                                                                            \
   if (v8) SCALAR_LAUNCH(RC_, true);                                                                                 \

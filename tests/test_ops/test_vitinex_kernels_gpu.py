@@ -120,7 +120,7 @@ def test_latent_kv_write(dtype, rank, R, dims):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,rank,R", [(8, 128, 64), (3, 40, 24), (5, 256, 64), (2, 512, 64), (4, 96, 16)])
+@pytest.mark.parametrize("H,rank,R", [(8, 128, 64), (3, 40, 24), (5, 256, 64), (2, 512, 64), (4, 96, 16), (3, 320, 32), (2, 44, 12), (2, 27, 6)])
 def test_attention_over_latent_view(dtype, H, rank, R):
     """Multi-query attention whose values are the leading channels of the keys (a view of the key pool)."""
     torch.manual_seed(7)
