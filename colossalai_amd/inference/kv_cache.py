@@ -29,6 +29,7 @@ class KVCacheManager:
         dtype=torch.bfloat16,
         layer_shapes: Optional[List[Optional[tuple]]] = None,
         layer_sources: Optional[List[Optional[int]]] = None,
+        layer_summaries: Optional[List[Optional[int]]] = None,
     ):
         """``layer_shapes`` (optional) gives each layer its own
         ``(kv_heads, key_dim, value_dim)`` or ``None`` for a layer that keeps no
@@ -37,7 +38,14 @@ class KVCacheManager:
         names, for a layer that projects no keys of its own, the layer whose
         pools it reads: ``k_pools[i]`` / ``v_pools[i]`` are then that layer's
         tensors (no second copy; the pages and page tables are shared by all
-        layers anyway), and the layer's own shape entry must be ``None``."""
+        layers anyway), and the layer's own shape entry must be ``None``.
+        ``layer_summaries`` (optional) gives, for a layer whose attention also reads
+        one mean key and value per block of ``P`` positions, that ``P``: the layer
+        gets a second, small pair of pools ``k_summaries[i]`` / ``v_summaries[i]``
+        ``[num_blocks, rows, Hkv, D]`` with ``rows = summary_rows_per_page(block_size, P)``;
+        summary ``b`` of a sequence lives in its page ``b // rows`` at row ``b % rows``,
+        so the sequence's page table addresses both pools and freeing its pages
+        frees its summaries."""
         assert block_size & (block_size - 1) == 0, "block_size must be a power of two"
         self.num_layers = num_layers
         self.block_size = block_size
@@ -63,6 +71,20 @@ class KVCacheManager:
                 assert self.layer_sources[src] is None and self.k_pools[src] is not None, \
                     f"layer {i} reads keys of layer {src}, which keeps none"
                 self.k_pools[i], self.v_pools[i] = self.k_pools[src], self.v_pools[src]
+        self.layer_summaries = list(layer_summaries) if layer_summaries is not None else [None] * num_layers
+        assert len(self.layer_summaries) == num_layers
+        self.k_summaries: List[Optional[torch.Tensor]] = [None] * num_layers
+        self.v_summaries: List[Optional[torch.Tensor]] = [None] * num_layers
+        for i, P in enumerate(self.layer_summaries):
+            if P is None:
+                continue
+            from ..ops.paged_attention import summary_rows_per_page
+
+            s = layer_shapes[i]
+            assert s is not None and P >= 1, f"layer {i} summarises keys it does not keep"
+            rows = summary_rows_per_page(block_size, int(P))
+            self.k_summaries[i] = torch.zeros(num_blocks, rows, s[0], s[1], device=self.device, dtype=dtype)
+            self.v_summaries[i] = torch.zeros(num_blocks, rows, s[0], s[2], device=self.device, dtype=dtype)
         self._free: List[int] = list(range(num_blocks - 1, -1, -1))
         self._tables: Dict[int, List[int]] = {}  # seq id -> block ids
 

@@ -58,9 +58,10 @@ class ContinuousBatchEngine:
             self.dtype = model.act_dtype
             shapes = model.kv_layer_shapes()
             sources = model.kv_layer_sources() if hasattr(model, "kv_layer_sources") else None
+            summaries = model.kv_layer_summaries() if hasattr(model, "kv_layer_summaries") else None
             self.kv = KVCacheManager(len(shapes), 0, 0, num_blocks=num_blocks, block_size=block_size,
                                      device=self.device, dtype=self.dtype, layer_shapes=shapes,
-                                     layer_sources=sources)
+                                     layer_sources=sources, layer_summaries=summaries)
             self.state = StateCacheManager(model.state_layer_buffers(), self.config.max_batch_size,
                                            device=self.device)
             self.rm = RequestManager(self.kv, max_batch_size=self.config.max_batch_size, state=self.state)

@@ -7,6 +7,7 @@ from .registry import load_pretrained, model_class_for, register_model, register
 from .kipirax import KipiraxConfig, KipiraxForCausalLM
 from .mubutar import MubutarConfig, MubutarForCausalLM
 from .vitinex import VitinexConfig, VitinexForCausalLM
+from .tarulix import TarulixConfig, TarulixForCausalLM
 from .llama import LLAMA_CONFIGS, LlamaConfig, LlamaForCausalLM, llama_flops_per_token
 from .bert import BERT_CONFIGS, BertConfig, BertForMaskedLM, BertForSequenceClassification
 from .opt import OPT_CONFIGS, OPTConfig, OPTForCausalLM
@@ -21,6 +22,7 @@ from .whisper import WHISPER_CONFIGS, WhisperConfig, WhisperForConditionalGenera
 
 __all__ = ["load_pretrained", "model_class_for", "register_model", "registered_models",
            "KipiraxConfig", "KipiraxForCausalLM", "MubutarConfig", "MubutarForCausalLM", "VitinexConfig", "VitinexForCausalLM",
+           "TarulixConfig", "TarulixForCausalLM",
            "LlamaConfig", "LlamaForCausalLM", "LLAMA_CONFIGS", "llama_flops_per_token",
            "OPTConfig", "OPTForCausalLM", "OPT_CONFIGS",
            "BertConfig", "BertForMaskedLM", "BertForSequenceClassification", "BERT_CONFIGS",

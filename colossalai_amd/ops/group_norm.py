@@ -27,7 +27,7 @@ from ._kernels import serving_kernels, use_serving_hip as use_hip
 __all__ = ["grouped_rms_norm", "grouped_rms_norm_ref", "head_rms_norm_gate", "head_rms_norm_gate_ref",
            "merge_rms_norm", "merge_rms_norm_ref", "add_rms_norm", "add_rms_norm_ref",
            "gated_grouped_rms_norm", "gated_grouped_rms_norm_ref", "layer_norm", "layer_norm_ref",
-           "add_layer_norm", "add_layer_norm_ref"]
+           "add_layer_norm", "add_layer_norm_ref", "add_scaled_unit_norm", "add_scaled_unit_norm_ref"]
 
 
 def grouped_rms_norm_ref(x, weight, groups: int, eps: float, residual=None, out_dtype=None):
@@ -147,3 +147,22 @@ def add_layer_norm(residual, y, w_out, mult: float, w_next, eps: float, out_dtyp
         return serving_kernels().add_layer_norm(residual, y.contiguous(), w_out, float(mult), w_next, eps,
                                                 out_dtype or y.dtype)
     return add_layer_norm_ref(residual, y, w_out, mult, w_next, eps, out_dtype)
+
+
+def add_scaled_unit_norm_ref(residual, a, b, scale_a: float, scale_b: float, gain: float, eps: float, out_dtype=None):
+    y = a.float() * scale_a if b is None else a.float() * scale_a + b.float() * scale_b
+    residual.add_(y / torch.sqrt((y * y).mean(-1, keepdim=True) + eps) * gain)
+    return residual.to(out_dtype) if out_dtype is not None else None
+
+
+def add_scaled_unit_norm(residual, a, b, scale_a: float, scale_b: float, gain: float, eps: float, out_dtype=None):
+    """Norm on a sublayer's *output*, with one number as its weight: ``y = scale_a * a (+ scale_b * b)``,
+    ``residual += gain * y / sqrt(mean(y^2) + eps)`` in place (float32 [N, W]; ``a``/``b`` sublayer outputs of any
+    activation type). With ``out_dtype`` the updated rows are also handed back in that type — the next sublayer's
+    input, when sublayers read the stream itself — in the same pass."""
+    if use_hip(residual):
+        assert residual.dtype == torch.float32 and residual.is_contiguous()
+        return serving_kernels().add_scaled_unit_norm(residual, a.contiguous(), None if b is None else b.contiguous(),
+                                                      float(scale_a), float(scale_b), float(gain), float(eps), out_dtype)
+    return add_scaled_unit_norm_ref(residual, a, b, scale_a, scale_b, gain, eps, out_dtype)
+
