@@ -315,5 +315,154 @@ void latent_kv_write(at::Tensor dkv, at::Tensor norm_w, double eps, at::Tensor f
   HIP_CHECK_LAST();
 }
 
+// --------------------------------------------- rotate-half rotary + weightless per-head RMS norm
+// One wave per (token, head): channel i < half pairs with channel i + half and turns by
+// positions[n] * freqs[i] (float32 angle); channels from 2 * half on pass. Then, with eps >= 0, the
+// head's vector is divided by sqrt(mean(x^2) + eps) over all D channels. The head's vector stays in
+// registers (D <= 64 * PER) between the two steps. x element (n, h, d) at n*xs + h*D + d; out dense.
+template <typename T, typename TO, int PER>
+__global__ __launch_bounds__(256) void rotate_halves_unit_norm_kernel(
+    TO* __restrict__ out, const T* __restrict__ x, long xs, const int* __restrict__ positions,
+    const float* __restrict__ freqs, long units, int H, int D, int half, float eps) {
+  const int lane = threadIdx.x & 63;
+  const long unit = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (unit >= units) return;
+  const long n = unit / H;
+  const int h = (int)(unit % H);
+  const T* src = x + n * xs + (long)h * D;
+  const float p = (float)positions[n];
+  float v[PER];
+  float ssq = 0.0f;
+#pragma unroll
+  for (int r = 0; r < PER; ++r) {
+    const int d = lane + 64 * r;
+    v[r] = 0.0f;
+    if (d < D) {
+      const float own = ldf(src + d);
+      if (d < 2 * half) {
+        const int i = d < half ? d : d - half;
+        const float other = ldf(src + (d < half ? d + half : d - half));
+        float sn, cs;
+        sincosf(p * freqs[i], &sn, &cs);
+        v[r] = d < half ? own * cs - other * sn : own * cs + other * sn;
+      } else {
+        v[r] = own;
+      }
+      ssq += v[r] * v[r];
+    }
+  }
+  float inv = 1.0f;
+  if (eps >= 0.0f) inv = 1.0f / sqrtf(wave_reduce_sum(ssq) / (float)D + eps);
+#pragma unroll
+  for (int r = 0; r < PER; ++r) {
+    const int d = lane + 64 * r;
+    if (d < D) stf(out + unit * D + d, v[r] * inv);
+  }
+}
+
+at::Tensor rotate_halves_unit_norm(at::Tensor x, at::Tensor positions, c10::optional<at::Tensor> freqs, double eps,
+                                   at::ScalarType out_dtype) {
+  check_act(x, "x");
+  TORCH_CHECK(x.dim() == 3 && x.stride(2) == 1 && (x.size(1) == 1 || x.stride(1) == x.size(2)),
+              "x must be [N, H, D] with the heads of a token side by side");
+  check_i32(positions, "positions");
+  const long N = x.size(0);
+  const int H = (int)x.size(1), D = (int)x.size(2);
+  TORCH_CHECK(positions.numel() == N && D <= 512, "head sizes up to 512");
+  int half = 0;
+  const float* fp = nullptr;
+  at::Tensor fr;
+  if (freqs.has_value() && freqs->numel() > 0) {
+    fr = *freqs;
+    TORCH_CHECK(fr.is_cuda() && is_f32(fr) && fr.is_contiguous() && 2 * fr.numel() <= D,
+                "freqs must be float32 [dims / 2] with dims <= D");
+    half = (int)fr.numel();
+    fp = fr.data_ptr<float>();
+  }
+  TORCH_CHECK(out_dtype == at::kFloat || out_dtype == at::kBFloat16);
+  at::Tensor out = at::empty({N, H, D}, x.options().dtype(out_dtype));
+  const long units = N * H;
+  if (units == 0) return out;
+  const dim3 grid((unsigned)((units + 3) / 4));
+#define RH_LAUNCH(PER_)                                                                                                 hipLaunchKernelGGL((rotate_halves_unit_norm_kernel<T, TO, PER_>), grid, dim3(256), 0, stream(), ptr<TO>(out),                           ptr<T>(x), (long)x.stride(0), positions.data_ptr<int>(), fp, units, H, D, half, (float)eps)
+  SERVING_DISPATCH_ACT(x, T, {
+    SERVING_DISPATCH_ACT(out, TO, {
+      if (D <= 64) RH_LAUNCH(1);
+      else if (D <= 128) RH_LAUNCH(2);
+      else if (D <= 256) RH_LAUNCH(4);
+      else RH_LAUNCH(8);
+    });
+  });
+#undef RH_LAUNCH
+  HIP_CHECK_LAST();
+  return out;
+}
+
+// ------------------------------------------------------------------ value mixing
+// out[n, c] = (1 - lam) * a[n, c] + lam * b[n, c], float32 inside, one rounding; rows may be strided.
+template <typename T>
+__global__ __launch_bounds__(256) void lerp_rows_kernel(T* __restrict__ out, const T* __restrict__ a, long as,
+                                                        const T* __restrict__ b, long bs, float lam, long N, int C) {
+  const long total = N * C;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    const long n = i / C;
+    const int c = (int)(i % C);
+    const float av = ldf(a + n * as + c), bv = ldf(b + n * bs + c);
+    stf(out + i, (1.0f - lam) * av + lam * bv);
+  }
+}
+
+at::Tensor lerp_rows(at::Tensor a, at::Tensor b, double lam) {
+  check_act(a, "a"); check_act(b, "b");
+  TORCH_CHECK(a.dim() == 2 && b.dim() == 2 && a.sizes() == b.sizes() && a.scalar_type() == b.scalar_type() &&
+              a.stride(1) == 1 && b.stride(1) == 1, "a and b must be [N, C] of one type with dense rows");
+  const long N = a.size(0);
+  const int C = (int)a.size(1);
+  at::Tensor out = at::empty({N, C}, a.options());
+  if (N * C == 0) return out;
+  SERVING_DISPATCH_ACT(a, T, {
+    hipLaunchKernelGGL(lerp_rows_kernel<T>, dim3(capped_grid((N * C + 255) / 256, 8192)), dim3(256), 0, stream(),
+                       ptr<T>(out), ptr<T>(a), (long)a.stride(0), ptr<T>(b), (long)b.stride(0), (float)lam, N, C);
+  });
+  HIP_CHECK_LAST();
+  return out;
+}
+
+// --------------------------------------------------------------- talking heads
+// o [N, H, G, Dv] float32 holds every query head's softmax weights applied to every key/value head's
+// values; mixing the weights of the heads is linear, so out[n, h, :] = sum_g talk[h, g] * o[n, g, kv(h), :]
+// with kv(h) = h / (H / G).
+template <typename TO>
+__global__ __launch_bounds__(256) void talk_mix_kernel(TO* __restrict__ out, const float* __restrict__ o,
+                                                       const float* __restrict__ talk, long N, int H, int G, int Dv) {
+  const long total = N * H * Dv;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    const int d = (int)(i % Dv);
+    const int h = (int)(i / Dv % H);
+    const long n = i / Dv / H;
+    const int c = h / (H / G);
+    float acc = 0.0f;
+    for (int g = 0; g < H; ++g) acc += talk[h * H + g] * o[((n * H + g) * G + c) * Dv + d];
+    stf(out + i, acc);
+  }
+}
+
+at::Tensor talk_mix(at::Tensor o, at::Tensor talk, at::ScalarType out_dtype) {
+  TORCH_CHECK(o.is_cuda() && is_f32(o) && o.dim() == 4 && o.is_contiguous(), "o must be contiguous float32 [N, H, G, Dv]");
+  const long N = o.size(0);
+  const int H = (int)o.size(1), G = (int)o.size(2), Dv = (int)o.size(3);
+  at::Tensor tk = f32c(talk);
+  TORCH_CHECK(tk.is_cuda() && tk.dim() == 2 && tk.size(0) == H && tk.size(1) == H && H % G == 0);
+  TORCH_CHECK(out_dtype == at::kFloat || out_dtype == at::kBFloat16);
+  at::Tensor out = at::empty({N, H, Dv}, o.options().dtype(out_dtype));
+  if (N == 0) return out;
+  SERVING_DISPATCH_ACT(out, TO, {
+    hipLaunchKernelGGL(talk_mix_kernel<TO>, dim3(capped_grid((N * H * Dv + 255) / 256, 8192)), dim3(256), 0, stream(),
+                       ptr<TO>(out), o.data_ptr<float>(), tk.data_ptr<float>(), N, H, G, Dv);
+  });
+  HIP_CHECK_LAST();
+  return out;
+}
+
 }  // namespace serving
 }  // namespace cai

@@ -177,8 +177,9 @@ DEV_INLINE void rows_dot(const T* __restrict__ x, const T* __restrict__ w, int K
   }
 }
 
-// block = (pair, chunk of 4 * R hidden rows): hidden[p, f] = relu(up_e[f, :] . h[n, :])^2
-template <typename T>
+// block = (pair, chunk of 4 * R hidden rows): hidden[p, f] = relu(up_e[f, :] . h[n, :])^2, or, GATED (the
+// expert's matrix stacks F gate rows on F up rows): hidden[p, f] = silu(gate_e[f, :] . h) * (up_e[f, :] . h)
+template <typename T, bool GATED>
 __global__ __launch_bounds__(256) void expert_up_gemv_kernel(
     T* __restrict__ hidden, const T* __restrict__ h, const T* __restrict__ w_up, const int* __restrict__ ids, int top,
     int E, int F, int W, int vec) {
@@ -191,11 +192,25 @@ __global__ __launch_bounds__(256) void expert_up_gemv_kernel(
   float acc[GEMV_R];
 #pragma unroll
   for (int r = 0; r < GEMV_R; ++r) acc[r] = 0.0f;
-  rows_dot<T, GEMV_R>(h + n * W, w_up + (long)e * F * W, W, row0, F, lane, vec, 1.0f, acc);
+  if constexpr (GATED) {
+    float up[GEMV_R];
 #pragma unroll
-  for (int r = 0; r < GEMV_R; ++r) {
-    const float v = fmaxf(wave_reduce_sum(acc[r]), 0.0f);
-    if (lane == 0 && row0 + r < F) stf(hidden + p * F + row0 + r, v * v);
+    for (int r = 0; r < GEMV_R; ++r) up[r] = 0.0f;
+    const T* we = w_up + (long)e * 2 * F * W;
+    rows_dot<T, GEMV_R>(h + n * W, we, W, row0, F, lane, vec, 1.0f, acc);
+    rows_dot<T, GEMV_R>(h + n * W, we + (long)F * W, W, row0, F, lane, vec, 1.0f, up);
+#pragma unroll
+    for (int r = 0; r < GEMV_R; ++r) {
+      const float g = wave_reduce_sum(acc[r]), u = wave_reduce_sum(up[r]);
+      if (lane == 0 && row0 + r < F) stf(hidden + p * F + row0 + r, g * sigmoidf_(g) * u);
+    }
+  } else {
+    rows_dot<T, GEMV_R>(h + n * W, w_up + (long)e * F * W, W, row0, F, lane, vec, 1.0f, acc);
+#pragma unroll
+    for (int r = 0; r < GEMV_R; ++r) {
+      const float v = fmaxf(wave_reduce_sum(acc[r]), 0.0f);
+      if (lane == 0 && row0 + r < F) stf(hidden + p * F + row0 + r, v * v);
+    }
   }
 }
 
@@ -205,17 +220,20 @@ template <typename T, typename TB>
 __global__ __launch_bounds__(256) void expert_down_gemv_kernel(
     float* __restrict__ out, const T* __restrict__ hidden, const T* __restrict__ w_down, const int* __restrict__ ids,
     const float* __restrict__ weights, const TB* __restrict__ base, const float* __restrict__ base_gate, long bgs,
-    int top, int E, int F, int W, int vec) {
+    int top, int E, int F, int W, int vec, const T* __restrict__ ident) {
+  // ident (the tokens' input rows [N, W], or null): an id >= E then names an identity expert and adds weight * ident[n]
   const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const long n = blockIdx.x;
   const int row0 = (blockIdx.y * 4 + wid) * GEMV_R;
   if (row0 >= W) return;
+  float idw = 0.0f;
   const float bscale = base_gate != nullptr ? sigmoidf_(base_gate[n * bgs]) : 1.0f;
   float acc[GEMV_R];
 #pragma unroll
   for (int r = 0; r < GEMV_R; ++r) acc[r] = 0.0f;
   for (int j = 0; j < top; ++j) {
     const int e = ids[n * top + j];
+    if (e >= E && ident != nullptr) idw += weights[n * top + j];
     if (e < 0 || e >= E) continue;
     rows_dot<T, GEMV_R>(hidden + (n * top + j) * F, w_down + (long)e * W * F, F, row0, W, lane, vec,
                         weights[n * top + j], acc);
@@ -225,13 +243,13 @@ __global__ __launch_bounds__(256) void expert_down_gemv_kernel(
     const float v = wave_reduce_sum(acc[r]);
     if (lane == 0 && row0 + r < W) {
       const long at = n * W + row0 + r;
-      out[at] = (base != nullptr ? ldf(base + at) * bscale : 0.0f) + v;
+      out[at] = (base != nullptr ? ldf(base + at) * bscale : 0.0f) + v + (ident != nullptr ? idw * ldf(ident + at) : 0.0f);
     }
   }
 }
 
 static void check_experts(const at::Tensor& h, const at::Tensor& w_up, const at::Tensor& w_down, const at::Tensor& ids,
-                          const at::Tensor& weights, const c10::optional<at::Tensor>& base) {
+                          const at::Tensor& weights, const c10::optional<at::Tensor>& base, bool gated = false) {
   check_act(h, "h");
   TORCH_CHECK(h.dim() == 2 && h.is_contiguous(), "h must be contiguous [N, W]");
   TORCH_CHECK(w_up.dim() == 3 && w_down.dim() == 3 && w_up.is_contiguous() && w_down.is_contiguous() && w_up.is_cuda() &&
@@ -239,7 +257,8 @@ static void check_experts(const at::Tensor& h, const at::Tensor& w_up, const at:
   TORCH_CHECK(w_up.scalar_type() == h.scalar_type() && w_down.scalar_type() == h.scalar_type(),
               "experts and their input share one dtype");
   TORCH_CHECK(w_up.size(2) == h.size(1) && w_down.size(0) == w_up.size(0) && w_down.size(1) == h.size(1) &&
-              w_down.size(2) == w_up.size(1), "expert matrix shapes do not fit [E, F, W] / [E, W, F]");
+              w_down.size(2) * (gated ? 2 : 1) == w_up.size(1),
+              "expert matrix shapes do not fit [E, F, W] (gated: [E, 2F, W]) / [E, W, F]");
   check_i32(ids, "ids");
   TORCH_CHECK(ids.dim() == 2 && ids.size(0) == h.size(0));
   TORCH_CHECK(weights.is_cuda() && is_f32(weights) && weights.is_contiguous() && weights.sizes() == ids.sizes(),
@@ -263,12 +282,13 @@ static const float* base_gate_ptr(const c10::optional<at::Tensor>& base_gate, co
 }
 
 at::Tensor expert_ffn_gemv(at::Tensor h, at::Tensor w_up, at::Tensor w_down, at::Tensor ids, at::Tensor weights,
-                           c10::optional<at::Tensor> base, c10::optional<at::Tensor> base_gate) {
-  check_experts(h, w_up, w_down, ids, weights, base);
+                           c10::optional<at::Tensor> base, c10::optional<at::Tensor> base_gate, bool gated,
+                           bool identity) {
+  check_experts(h, w_up, w_down, ids, weights, base, gated);
   long bgs = 0;
   const float* bgp = base_gate_ptr(base_gate, base, h.size(0), &bgs);
   const long N = h.size(0);
-  const int W = (int)h.size(1), E = (int)w_up.size(0), F = (int)w_up.size(1), top = (int)ids.size(1);
+  const int W = (int)h.size(1), E = (int)w_up.size(0), F = (int)w_down.size(2), top = (int)ids.size(1);
   at::Tensor out = at::empty({N, W}, h.options().dtype(at::kFloat));
   if (N == 0) return out;
   at::Tensor hidden = at::empty({N * top, F}, h.options());
@@ -278,20 +298,25 @@ at::Tensor expert_ffn_gemv(at::Tensor h, at::Tensor w_up, at::Tensor w_down, at:
   const int vec_up = (W % 8 == 0 && aligned(h) && aligned(w_up)) ? 1 : 0;
   const int vec_down = (F % 8 == 0 && aligned(hidden) && aligned(w_down)) ? 1 : 0;
   SERVING_DISPATCH_ACT(h, T, {
-    hipLaunchKernelGGL(expert_up_gemv_kernel<T>, dim3((unsigned)(N * top), (unsigned)((F + rows_per_block - 1) / rows_per_block)),
-                       dim3(256), 0, stream(), ptr<T>(hidden), ptr<T>(h), ptr<T>(w_up), ids.data_ptr<int>(), top, E, F, W,
-                       vec_up);
+    const dim3 up_grid((unsigned)(N * top), (unsigned)((F + rows_per_block - 1) / rows_per_block));
+    if (gated)
+      hipLaunchKernelGGL((expert_up_gemv_kernel<T, true>), up_grid, dim3(256), 0, stream(), ptr<T>(hidden), ptr<T>(h),
+                         ptr<T>(w_up), ids.data_ptr<int>(), top, E, F, W, vec_up);
+    else
+      hipLaunchKernelGGL((expert_up_gemv_kernel<T, false>), up_grid, dim3(256), 0, stream(), ptr<T>(hidden), ptr<T>(h),
+                         ptr<T>(w_up), ids.data_ptr<int>(), top, E, F, W, vec_up);
+    const T* idp = identity ? ptr<T>(h) : (const T*)nullptr;
     const dim3 grid((unsigned)N, (unsigned)((W + rows_per_block - 1) / rows_per_block));
     if (base.has_value()) {
       SERVING_DISPATCH_ACT(*base, TB, {
         hipLaunchKernelGGL((expert_down_gemv_kernel<T, TB>), grid, dim3(256), 0, stream(), out.data_ptr<float>(),
                            ptr<T>(hidden), ptr<T>(w_down), ids.data_ptr<int>(), weights.data_ptr<float>(), ptr<TB>(*base),
-                           bgp, bgs, top, E, F, W, vec_down);
+                           bgp, bgs, top, E, F, W, vec_down, idp);
       });
     } else {
       hipLaunchKernelGGL((expert_down_gemv_kernel<T, float>), grid, dim3(256), 0, stream(), out.data_ptr<float>(),
                          ptr<T>(hidden), ptr<T>(w_down), ids.data_ptr<int>(), weights.data_ptr<float>(),
-                         (const float*)nullptr, (const float*)nullptr, 0L, top, E, F, W, vec_down);
+                         (const float*)nullptr, (const float*)nullptr, 0L, top, E, F, W, vec_down, idp);
     }
   });
   HIP_CHECK_LAST();
@@ -304,9 +329,16 @@ at::Tensor expert_ffn_gemv(at::Tensor h, at::Tensor w_up, at::Tensor w_down, at:
 template <typename T, typename TB, bool VEC>
 __global__ __launch_bounds__(256) void expert_combine_kernel(
     float* __restrict__ out, const T* __restrict__ y, const int* __restrict__ inv, const float* __restrict__ weights,
-    const TB* __restrict__ base, const float* __restrict__ base_gate, long bgs, int top, int W, long rows) {
+    const TB* __restrict__ base, const float* __restrict__ base_gate, long bgs, int top, int W, long rows,
+    const int* __restrict__ ids, int E, const T* __restrict__ ident) {
+  // ident (the tokens' input rows [N, W], with ids [N, top] and the number E of real experts; or null): a pair whose
+  // id is >= E names an identity expert, has no row in y and adds weight * ident[n]
   const long n = blockIdx.x;
   const float bscale = base_gate != nullptr ? sigmoidf_(base_gate[n * bgs]) : 1.0f;
+  float idw = 0.0f;
+  if (ident != nullptr)
+    for (int j = 0; j < top; ++j)
+      if (ids[n * top + j] >= E) idw += weights[n * top + j];
   if (VEC) {
     for (int w = threadIdx.x * 8; w < W; w += blockDim.x * 8) {
       float acc[8];
@@ -318,9 +350,15 @@ __global__ __launch_bounds__(256) void expert_combine_kernel(
 #pragma unroll
         for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
       }
+      if (ident != nullptr) {
+        float v[8];
+        load8(ident + n * W + w, v);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] += idw * v[e];
+      }
       for (int j = 0; j < top; ++j) {
         const long r = inv[n * top + j];
-        if (r >= 0 && r < rows) {
+        if (r >= 0 && r < rows && (ident == nullptr || ids[n * top + j] < E)) {
           float v[8];
           load8(y + r * W + w, v);
           const float wj = weights[n * top + j];
@@ -333,9 +371,11 @@ __global__ __launch_bounds__(256) void expert_combine_kernel(
   } else {
     for (int w = threadIdx.x; w < W; w += blockDim.x) {
       float acc = base != nullptr ? ldf(base + n * W + w) * bscale : 0.0f;
+      if (ident != nullptr) acc += idw * ldf(ident + n * W + w);
       for (int j = 0; j < top; ++j) {
         const long r = inv[n * top + j];
-        if (r >= 0 && r < rows) acc += weights[n * top + j] * ldf(y + r * W + w);
+        if (r >= 0 && r < rows && (ident == nullptr || ids[n * top + j] < E))
+          acc += weights[n * top + j] * ldf(y + r * W + w);
       }
       out[n * W + w] = acc;
     }
@@ -343,7 +383,8 @@ __global__ __launch_bounds__(256) void expert_combine_kernel(
 }
 
 at::Tensor expert_combine(at::Tensor y, at::Tensor inv, at::Tensor weights, c10::optional<at::Tensor> base,
-                          c10::optional<at::Tensor> base_gate) {
+                          c10::optional<at::Tensor> base_gate, c10::optional<at::Tensor> ids, int64_t num_experts,
+                          c10::optional<at::Tensor> identity_rows) {
   check_act(y, "y");
   check_i32(inv, "inv");
   TORCH_CHECK(y.dim() == 2 && y.is_contiguous() && inv.dim() == 2 && inv.size(0) * inv.size(1) == y.size(0),
@@ -357,21 +398,34 @@ at::Tensor expert_combine(at::Tensor y, at::Tensor inv, at::Tensor weights, c10:
   }
   long bgs = 0;
   const float* bgp = base_gate_ptr(base_gate, base, N, &bgs);
+  const int* idsp = nullptr;
+  const void* identp = nullptr;
+  if (identity_rows.has_value()) {
+    TORCH_CHECK(ids.has_value(), "identity experts are told from real ones by their ids");
+    check_i32(*ids, "ids");
+    TORCH_CHECK(ids->sizes() == inv.sizes() && identity_rows->is_cuda() && identity_rows->is_contiguous() &&
+                identity_rows->dim() == 2 && identity_rows->size(0) == N && identity_rows->size(1) == W &&
+                identity_rows->scalar_type() == y.scalar_type(), "identity rows must be contiguous [N, W] of y's type");
+    idsp = ids->data_ptr<int>();
+    identp = identity_rows->data_ptr();
+  }
+  const int E = (int)num_experts;
   at::Tensor out = at::empty({N, W}, y.options().dtype(at::kFloat));
   if (N == 0) return out;
   auto al32 = [](const at::Tensor& t) { return reinterpret_cast<uintptr_t>(t.data_ptr()) % 32 == 0; };
-  const bool vec = W % 8 == 0 && al32(y) && al32(out) && (!base.has_value() || al32(*base));
+  const bool vec = W % 8 == 0 && al32(y) && al32(out) && (!base.has_value() || al32(*base)) &&
+                   (!identity_rows.has_value() || al32(*identity_rows));
   const float* nobase = nullptr;
 #define COMBINE_LAUNCH(TB_, bp)                                                                                       \
   do {                                                                                                                \
     if (vec)                                                                                                          \
       hipLaunchKernelGGL((expert_combine_kernel<T, TB_, true>), dim3((unsigned)N), dim3(256), 0, stream(),           \
                          out.data_ptr<float>(), ptr<T>(y), inv.data_ptr<int>(), weights.data_ptr<float>(), bp, bgp,  \
-                         bgs, top, W, (long)y.size(0));                                                               \
+                         bgs, top, W, (long)y.size(0), idsp, E, (const T*)identp);                                    \
     else                                                                                                              \
       hipLaunchKernelGGL((expert_combine_kernel<T, TB_, false>), dim3((unsigned)N), dim3(256), 0, stream(),          \
                          out.data_ptr<float>(), ptr<T>(y), inv.data_ptr<int>(), weights.data_ptr<float>(), bp, bgp,  \
-                         bgs, top, W, (long)y.size(0));                                                               \
+                         bgs, top, W, (long)y.size(0), idsp, E, (const T*)identp);                                    \
   } while (0)
   SERVING_DISPATCH_ACT(y, T, {
     if (base.has_value()) {

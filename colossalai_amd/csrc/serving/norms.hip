@@ -559,5 +559,91 @@ c10::optional<at::Tensor> add_layer_norm(c10::optional<at::Tensor> residual, at:
   return out;
 }
 
+// ------------------------------------------- norm on a sublayer's output, one number as weight
+// One block per row: y = sa * a (+ sb * b); residual += gain * y / sqrt(mean(y^2) + eps) (float32,
+// in place); with `cast` the updated row is also stored in an activation type — the next
+// sublayer's input when sublayers read the stream itself. The row's y stays in registers
+// (W <= 256 * PER) between the reduction and the update.
+template <typename TA, typename TB, typename TO, int PER>
+__global__ __launch_bounds__(256) void add_scaled_unit_norm_kernel(
+    TO* __restrict__ cast, float* __restrict__ residual, const TA* __restrict__ a, const TB* __restrict__ b, float sa,
+    float sb, float gain, int W, float eps) {
+  __shared__ float red[8];
+  const long row = blockIdx.x;
+  float y[PER];
+  float ssq = 0.0f;
+#pragma unroll
+  for (int r = 0; r < PER; ++r) {
+    const int i = threadIdx.x + 256 * r;
+    y[r] = 0.0f;
+    if (i < W) {
+      y[r] = sa * ldf(a + row * W + i);
+      if (b != nullptr) y[r] += sb * ldf(b + row * W + i);
+      ssq += y[r] * y[r];
+    }
+  }
+  ssq = block_reduce_sum(ssq, red);
+  const float f = gain / sqrtf(ssq / (float)W + eps);
+#pragma unroll
+  for (int r = 0; r < PER; ++r) {
+    const int i = threadIdx.x + 256 * r;
+    if (i < W) {
+      const float v = residual[row * W + i] + f * y[r];
+      residual[row * W + i] = v;
+      if (cast != nullptr) stf(cast + row * W + i, v);
+    }
+  }
+}
+
+c10::optional<at::Tensor> add_scaled_unit_norm(at::Tensor residual, at::Tensor a, c10::optional<at::Tensor> b,
+                                               double scale_a, double scale_b, double gain, double eps,
+                                               c10::optional<at::ScalarType> out_dtype) {
+  TORCH_CHECK(residual.is_cuda() && is_f32(residual) && residual.dim() == 2 && residual.is_contiguous(),
+              "residual must be contiguous float32 [N, W]");
+  check_act(a, "a");
+  TORCH_CHECK(a.is_contiguous() && a.sizes() == residual.sizes(), "a must be contiguous and of the residual's shape");
+  if (b.has_value()) {
+    check_act(*b, "b");
+    TORCH_CHECK(b->is_contiguous() && b->sizes() == residual.sizes(), "b must be contiguous and of the residual's shape");
+  }
+  const long N = residual.size(0);
+  const int W = (int)residual.size(1);
+  TORCH_CHECK(W <= 256 * 64, "rows of up to 16384 elements");
+  at::Tensor out;
+  if (out_dtype.has_value()) {
+    TORCH_CHECK(*out_dtype == at::kFloat || *out_dtype == at::kBFloat16);
+    out = at::empty({N, W}, residual.options().dtype(*out_dtype));
+  }
+  if (N > 0) {
+    const at::Tensor like = out_dtype.has_value() ? out : residual;
+    const float* nob = nullptr;
+#define ASUN_LAUNCH(TB_, BP_, PER_)                                                                                     \
+  hipLaunchKernelGGL((add_scaled_unit_norm_kernel<TA, TB_, TO, PER_>), dim3((unsigned)N), dim3(256), 0, stream(), op,   \
+                     residual.data_ptr<float>(), ptr<TA>(a), BP_, (float)scale_a, (float)scale_b, (float)gain, W,       \
+                     (float)eps)
+#define ASUN_SIZES(TB_, BP_)                     \
+  do {                                           \
+    if (W <= 1024) ASUN_LAUNCH(TB_, BP_, 4);     \
+    else if (W <= 4096) ASUN_LAUNCH(TB_, BP_, 16); \
+    else ASUN_LAUNCH(TB_, BP_, 64);              \
+  } while (0)
+    SERVING_DISPATCH_ACT(a, TA, {
+      SERVING_DISPATCH_ACT(like, TO, {
+        TO* op = out_dtype.has_value() ? ptr<TO>(out) : (TO*)nullptr;
+        if (b.has_value()) {
+          SERVING_DISPATCH_ACT(*b, TB, { ASUN_SIZES(TB, ptr<TB>(*b)); });
+        } else {
+          ASUN_SIZES(float, nob);
+        }
+      });
+    });
+#undef ASUN_SIZES
+#undef ASUN_LAUNCH
+    HIP_CHECK_LAST();
+  }
+  if (!out_dtype.has_value()) return c10::nullopt;
+  return out;
+}
+
 }  // namespace serving
 }  // namespace cai

@@ -1,7 +1,10 @@
 // Attention of a ragged batch over paged keys/values with a sliding window,
 // kept first tokens, a linear distance penalty, a per-head output gate, a tanh
 // soft cap on the scaled score and an optional sink (one more place of score 0
-// in the softmax denominator that carries no value).
+// in the softmax denominator that carries no value; with sink logits its score is learned per
+// head), an additive per-distance table, block summaries (one mean key/value per block of
+// positions that lies wholly before the window, kept in a small pool of their own) and, for
+// talking heads, every query head's weights applied to every key/value head's values.
 //
 // One wave per (token, query head). The visible keys of a token are two
 // position ranges: the kept prefix [0, min(keep_first, lo)) and the window
@@ -50,7 +53,14 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
     const T* __restrict__ vpool, const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ tok_seq,
     const int* __restrict__ positions, const float* __restrict__ slopes, const T* __restrict__ gate, long gate_stride,
     int H, int G, int D, int Dv, int page_shift, float scale, int window, int keep_first, int kvec, int vvec,
-    float softcap, int sink, long vrow, long vhead) {
+    float softcap, int sink, long vrow, long vhead, const float* __restrict__ sink_logits,
+    const float* __restrict__ dist_bias, int dist_rows, const T* __restrict__ ksum, const T* __restrict__ vsum,
+    int sum_shift, int sum_block, float* __restrict__ cross_out) {
+  // sink_logits [H]: the sink's score per head instead of 0. dist_bias [dist_rows, H]: added to the score of a key at
+  // distance d (row min(d, dist_rows - 1)). ksum / vsum: block summaries, rows [pages << sum_shift]; a query at
+  // `pos` sees the first max(0, (pos - window + 1) / sum_block) of its sequence's, ahead of its other keys and
+  // without distance terms. cross_out [N, H, G, Dv] float32: the grid then has G blocks per (token, kv head, chunk),
+  // block c applies the heads' weights to the values of kv head c.
   // vrow / vhead: elements between the value rows of neighbouring pool rows / kv heads (G * Dv and Dv for a
   // pool of its own; a value pool that is a view into wider rows, e.g. the leading channels of the keys, has others)
   extern __shared__ __align__(16) float lds[];
@@ -61,9 +71,12 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
   float* pw = lds + RC * Dp + wid * (RC * 64 + 64);       // [RC][64] scores, then weights, of this wave's key block
   int* prow = reinterpret_cast<int*>(pw + RC * 64);       // [64] pool rows of the block
   float* part = lds + RC * Dp + nw * (RC * 64 + 64);      // [waves][RC][2 + Dv] partial states
-  const long n = blockIdx.x / (G * chunks);
-  const int g = (int)(blockIdx.x / chunks) % G;
-  const int h0 = g * R + (int)(blockIdx.x % chunks) * RC;  // first query head of this block
+  const int VC = cross_out != nullptr ? G : 1;
+  const long bx = blockIdx.x / VC;
+  const long n = bx / (G * chunks);
+  const int g = (int)(bx / chunks) % G;
+  const int vg = cross_out != nullptr ? (int)(blockIdx.x % VC) : g;  // kv head whose values this block reads
+  const int h0 = g * R + (int)(bx % chunks) * RC;  // first query head of this block
   const int nh = min(RC, g * R + R - h0);
   const int b = tok_seq[n];
   const int pos = positions[n];
@@ -80,7 +93,9 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
   for (int r = 0; r < RC; ++r) slope[r] = (slopes != nullptr && r < nh) ? slopes[h0 + r] : 0.0f;
 
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-  const int n_keep = window > 0 ? min(keep_first, lo) : 0;
+  const int n_sum = (ksum != nullptr && window > 0) ? max(0, (pos - window + 1) / sum_block) : 0;
+  const int sum_mask = (1 << sum_shift) - 1;
+  const int n_keep = (window > 0 ? min(keep_first, lo) : 0) + n_sum;  // summaries, then kept first tokens
   const int total = n_keep + (pos - lo + 1);
   const float inv_cap = softcap > 0.0f ? 1.0f / softcap : 0.0f;
   const int part8 = lane & 7, ksub = lane >> 3;
@@ -108,12 +123,14 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
     auto score_step = [&](int sub) {
       const int idx = base + sub * 8 + ksub;
       const bool valid = idx < total;
-      const int j = valid ? (idx < n_keep ? idx : lo + (idx - n_keep)) : pos;
-      const int row = (bt[j >> page_shift] << page_shift) + (j & page_mask);
+      const bool summary = valid && idx < n_sum;
+      const int j = valid ? (idx < n_keep ? idx - n_sum : lo + (idx - n_keep)) : pos;
+      const int row = summary ? (bt[idx >> sum_shift] << sum_shift) + (idx & sum_mask)
+                              : (bt[j >> page_shift] << page_shift) + (j & page_mask);
       float dots[RC];
 #pragma unroll
       for (int r = 0; r < RC; ++r) dots[r] = 0.0f;
-      const T* kr = kpool + ((long)row * G + g) * D;
+      const T* kr = (summary ? ksum : kpool) + ((long)row * G + g) * D;
       if (kvec) {
         for (int d = d_lo; d < d_hi; d += 8) {
           float kv[8];
@@ -140,9 +157,13 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
         for (int r = 0; r < RC; ++r) {
           float sc = dots[r] * scale;
           if (softcap > 0.0f) sc = softcap * tanhf(sc * inv_cap);
-          pw[r * 64 + sub * 8 + ksub] = valid ? sc - slope[r] * (float)(pos - j) : -INFINITY;
+          if (!summary) {
+            sc -= slope[r] * (float)(pos - j);
+            if (dist_bias != nullptr && r < nh) sc += dist_bias[(long)min(pos - j, dist_rows - 1) * H + h0 + r];
+          }
+          pw[r * 64 + sub * 8 + ksub] = valid ? sc : -INFINITY;
         }
-        prow[sub * 8 + ksub] = row;
+        prow[sub * 8 + ksub] = summary ? -1 - row : row;  // a summary row is marked by its sign
       }
     };
     if (cnt == 64) {  // straight-line: all eight steps' lookups and key loads issue before the first product
@@ -174,7 +195,8 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
       for (int jj = vsub; jj < cnt; jj += vks) {
         float v[8];
         if (vlive) {
-          load8(vpool + (long)prow[jj] * vrow + (long)g * vhead + vch, v);
+          const int pr = prow[jj];
+          load8((pr < 0 ? vsum : vpool) + (long)(pr < 0 ? -1 - pr : pr) * vrow + (long)vg * vhead + vch, v);
         } else {
 #pragma unroll
           for (int e = 0; e < 8; ++e) v[e] = 0.0f;
@@ -190,7 +212,8 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
     const int dva = 2 * lane, dvb = 128 + 2 * lane;
 #pragma unroll 8
     for (int jj = 0; jj < cnt; ++jj) {
-      const T* vr = vpool + (long)prow[jj] * vrow + (long)g * vhead;
+      const int pr = prow[jj];
+      const T* vr = (pr < 0 ? vsum : vpool) + (long)(pr < 0 ? -1 - pr : pr) * vrow + (long)vg * vhead;
       float v0 = 0.0f, v1 = 0.0f, v2 = 0.0f, v3 = 0.0f;
       if (vvec) {
         if (dva < Dv) load2(vr + dva, v0, v1);
@@ -244,10 +267,17 @@ __global__ __launch_bounds__(64 * ATT_WAVES) void paged_attention_kernel(
         o += part[(w * RC + r) * PS + 2 + dv] * f;
       }
     }
-    if (sink) ll += expf(-mm);  // the sink's score is 0
+    if (sink_logits != nullptr) {  // a learned score: it may be the largest of the row
+      const float sk = sink_logits[h0 + r], m2 = fmaxf(mm, sk), f2 = expf(mm - m2);
+      ll = ll * f2 + expf(sk - m2);
+      o *= f2;
+    } else if (sink) {
+      ll += expf(-mm);  // the sink's score is 0
+    }
     float scale_out = 1.0f / ll;
     if (gate != nullptr) scale_out *= sigmoidf_(ldf(gate + n * gate_stride + h0 + r));
-    stf(out + (n * H + h0 + r) * (long)Dv + dv, o * scale_out);
+    if (cross_out != nullptr) cross_out[((n * H + h0 + r) * G + vg) * (long)Dv + dv] = o * scale_out;
+    else stf(out + (n * H + h0 + r) * (long)Dv + dv, o * scale_out);
   }
 }
 
@@ -545,6 +575,66 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     }
 }
 
+// What the split-key kernel takes beyond the common parameters (all optional).
+struct ScalarExtras {
+  const float* sink_logits = nullptr;
+  const float* dist_bias = nullptr;
+  int dist_rows = 0;
+  const void* ksum = nullptr;
+  const void* vsum = nullptr;
+  int sum_shift = 0, sum_block = 1;
+  float* cross_out = nullptr;
+};
+
+static void launch_scalar_attention(at::Tensor& out, const at::Tensor& q, const at::Tensor& kpool, const at::Tensor& vpool,
+                                    const at::Tensor& block_tables, const at::Tensor& tok_seq, const at::Tensor& positions,
+                                    const float* slp, const c10::optional<at::Tensor>& gate, long gstride, double scale,
+                                    int64_t window, int64_t keep_first, double softcap, bool sink, int page_shift,
+                                    long vrow, long vhead, const ScalarExtras& x) {
+  const long N = q.size(0);
+  const int H = (int)q.size(1), D = (int)q.size(2);
+  const int G = (int)kpool.size(2), Dv = (int)vpool.size(3);
+  const int VC = x.cross_out != nullptr ? G : 1;
+  const int Dp = (D + 7) & ~7;
+  const int R = H / G;
+  int rc = RC_MAX;
+  while (rc > 1 && (rc > R || N * G * VC * ((R + rc - 1) / rc) < 256)) rc >>= 1;  // enough blocks to cover the CUs
+  auto lds_bytes = [&](int nw) { return (size_t)(rc * Dp + nw * (rc * 64 + 64) + nw * rc * (2 + Dv)) * sizeof(float); };
+  // wide value rows (a latent of several hundred channels): fewer waves, then fewer heads per block
+  int nwaves = ATT_WAVES;
+  while (lds_bytes(nwaves) > 64 * 1024 && nwaves > 4) nwaves >>= 1;
+  while (lds_bytes(nwaves) > 64 * 1024 && rc > 1) rc >>= 1;
+  const int chunks = (R + rc - 1) / rc;
+  const size_t smem = lds_bytes(nwaves);
+  TORCH_CHECK(smem <= 64 * 1024, "head sizes too large for the scalar attention kernel");
+  const int kvec = D % 8 == 0 ? 1 : 0;   // 16-byte (bfloat16) / 32-byte (float32) aligned key slices
+  const int vvec_even = Dv % 2 == 0 ? 1 : 0;
+  // value rows of a multiple of 8 channels whose loads are aligned take the 8-channels-per-lane value phase
+  const bool v8 = Dv >= 8 && Dv % 8 == 0 && reinterpret_cast<uintptr_t>(vpool.data_ptr()) % 32 == 0 &&
+                  vrow % 8 == 0 && vhead % 8 == 0;
+  TORCH_CHECK(v8 || Dv <= 256, "value rows above 256 channels must be a multiple of 8 channels and aligned");
+  const int vvec_ok = (vrow % 2 == 0 && vhead % 2 == 0) ? 1 : 0;
+#define SCALAR_CASE(RC_)                                                                                            \
+  if (v8) SCALAR_LAUNCH(RC_, true);                                                                                 \
+  else SCALAR_LAUNCH(RC_, false)
+#define SCALAR_LAUNCH(RC_, V8_)                                                                                     \
+  hipLaunchKernelGGL((paged_attention_kernel<T, RC_, V8_>), dim3((unsigned)(N * G * chunks * VC)), dim3(64 * nwaves), smem,   \
+                     stream(), x.cross_out != nullptr ? (T*)nullptr : ptr<T>(out), ptr<T>(q), (long)q.stride(0), ptr<T>(kpool), ptr<T>(vpool),             \
+                     block_tables.data_ptr<int>(), (int)block_tables.stride(0), tok_seq.data_ptr<int>(),            \
+                     positions.data_ptr<int>(), slp, gate.has_value() ? ptr<T>(*gate) : (const T*)nullptr, gstride, \
+                     H, G, D, Dv, page_shift, (float)scale, (int)window, (int)keep_first, kvec,                      \
+                     vvec_even & vvec_ok, (float)softcap, sink ? 1 : 0, vrow, vhead, x.sink_logits, x.dist_bias, x.dist_rows,      \
+                     (const T*)x.ksum, (const T*)x.vsum, x.sum_shift, x.sum_block, x.cross_out)
+  SERVING_DISPATCH_ACT(q, T, {
+    if (rc == 4) { SCALAR_CASE(4); }
+    else if (rc == 2) { SCALAR_CASE(2); }
+    else { SCALAR_CASE(1); }
+  });
+#undef SCALAR_CASE
+#undef SCALAR_LAUNCH
+  HIP_CHECK_LAST();
+}
+
 at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at::Tensor block_tables, at::Tensor cu,
                            at::Tensor start, at::Tensor tok_seq, at::Tensor positions, double scale, int64_t window,
                            int64_t keep_first, c10::optional<at::Tensor> slopes, c10::optional<at::Tensor> gate,
@@ -626,44 +716,141 @@ at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at:
     HIP_CHECK_LAST();
     return out;
   }
-  const int Dp = (D + 7) & ~7;
-  const int R = H / G;
-  int rc = RC_MAX;
-  while (rc > 1 && (rc > R || N * G * ((R + rc - 1) / rc) < 256)) rc >>= 1;  // enough blocks to cover the CUs
-  auto lds_bytes = [&](int nw) { return (size_t)(rc * Dp + nw * (rc * 64 + 64) + nw * rc * (2 + Dv)) * sizeof(float); };
-  // wide value rows (a latent of several hundred channels): fewer waves, then fewer heads per block
-  int nwaves = ATT_WAVES;
-  while (lds_bytes(nwaves) > 64 * 1024 && nwaves > 4) nwaves >>= 1;
-  while (lds_bytes(nwaves) > 64 * 1024 && rc > 1) rc >>= 1;
-  const int chunks = (R + rc - 1) / rc;
-  const size_t smem = lds_bytes(nwaves);
-  TORCH_CHECK(smem <= 64 * 1024, "head sizes too large for the scalar attention kernel");
-  const int kvec = D % 8 == 0 ? 1 : 0;   // 16-byte (bfloat16) / 32-byte (float32) aligned key slices
-  const int vvec_even = Dv % 2 == 0 ? 1 : 0;
-  // value rows of a multiple of 8 channels whose loads are aligned take the 8-channels-per-lane value phase
-  const bool v8 = Dv >= 8 && Dv % 8 == 0 && reinterpret_cast<uintptr_t>(vpool.data_ptr()) % 32 == 0 &&
-                  vrow % 8 == 0 && vhead % 8 == 0;
-  TORCH_CHECK(v8 || Dv <= 256, "value rows above 256 channels must be a multiple of 8 channels and aligned");
-  const int vvec_ok = (vrow % 2 == 0 && vhead % 2 == 0) ? 1 : 0;
-#define SCALAR_CASE(RC_)                                                                                            \
-  if (v8) SCALAR_LAUNCH(RC_, true);                                                                                 \
-  else SCALAR_LAUNCH(RC_, false)
-#define SCALAR_LAUNCH(RC_, V8_)                                                                                     \
-  hipLaunchKernelGGL((paged_attention_kernel<T, RC_, V8_>), dim3((unsigned)(N * G * chunks)), dim3(64 * nwaves), smem,   \
-                     stream(), ptr<T>(out), ptr<T>(q), (long)q.stride(0), ptr<T>(kpool), ptr<T>(vpool),             \
-                     block_tables.data_ptr<int>(), (int)block_tables.stride(0), tok_seq.data_ptr<int>(),            \
-                     positions.data_ptr<int>(), slp, gate.has_value() ? ptr<T>(*gate) : (const T*)nullptr, gstride, \
-                     H, G, D, Dv, page_shift, (float)scale, (int)window, (int)keep_first, kvec,                      \
-                     vvec_even & vvec_ok, (float)softcap, sink ? 1 : 0, vrow, vhead)
-  SERVING_DISPATCH_ACT(q, T, {
-    if (rc == 4) { SCALAR_CASE(4); }
-    else if (rc == 2) { SCALAR_CASE(2); }
-    else { SCALAR_CASE(1); }
-  });
-#undef SCALAR_CASE
-#undef SCALAR_LAUNCH
-  HIP_CHECK_LAST();
+  launch_scalar_attention(out, q, kpool, vpool, block_tables, tok_seq, positions, slp, gate, gstride, scale, window,
+                          keep_first, softcap, sink, page_shift, vrow, vhead, ScalarExtras());
   return out;
+}
+
+// The split-key kernel with its optional extras, for prompt portions and decode tokens alike: a learned sink per
+// head, a per-distance bias table, block summaries ahead of the window, and (cross) every query head's weights
+// applied to every kv head's values, returned as float32 [N, H, G, Dv] for a talking-heads mix.
+at::Tensor paged_attention_ext(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at::Tensor block_tables,
+                               at::Tensor tok_seq, at::Tensor positions, double scale, int64_t window,
+                               int64_t keep_first, c10::optional<at::Tensor> slopes, c10::optional<at::Tensor> gate,
+                               double softcap, bool sink, c10::optional<at::Tensor> sink_logits,
+                               c10::optional<at::Tensor> dist_bias, c10::optional<at::Tensor> ksum,
+                               c10::optional<at::Tensor> vsum, int64_t sum_block, bool cross) {
+  check_act(q, "q");
+  TORCH_CHECK(softcap >= 0.0, "softcap must not be negative (0 = none)");
+  TORCH_CHECK(q.dim() == 3 && q.stride(2) == 1 && q.stride(1) == q.size(2), "q must be [N, H, D] with dense rows");
+  TORCH_CHECK(kpool.dim() == 4 && vpool.dim() == 4 && kpool.is_contiguous() && vpool.is_contiguous(),
+              "pools must be contiguous [pages, page, G, D]");
+  TORCH_CHECK(kpool.scalar_type() == q.scalar_type() && vpool.scalar_type() == q.scalar_type(),
+              "query and pools share one dtype");
+  const long N = q.size(0);
+  const int H = (int)q.size(1), D = (int)q.size(2);
+  const int page = (int)kpool.size(1), G = (int)kpool.size(2), Dv = (int)vpool.size(3);
+  TORCH_CHECK(kpool.size(3) == D && vpool.size(2) == G && vpool.size(1) == page && vpool.size(0) == kpool.size(0));
+  TORCH_CHECK(H % G == 0 && Dv <= 512 && page > 0 && (page & (page - 1)) == 0);
+  check_i32(block_tables, "block_tables"); check_i32(tok_seq, "tok_seq"); check_i32(positions, "positions");
+  TORCH_CHECK(block_tables.dim() == 2 && tok_seq.numel() == N && positions.numel() == N);
+  TORCH_CHECK(window >= 0 && keep_first >= 0);
+  int page_shift = 0;
+  while ((1 << page_shift) < page) ++page_shift;
+  at::Tensor sl, sk, db;
+  const float* slp = nullptr;
+  if (slopes.has_value()) {
+    sl = f32c(*slopes);
+    TORCH_CHECK(sl.numel() == H);
+    slp = sl.data_ptr<float>();
+  }
+  long gstride = 0;
+  if (gate.has_value()) {
+    TORCH_CHECK(gate->scalar_type() == q.scalar_type() && gate->dim() == 2 && gate->size(0) == N &&
+                gate->size(1) == H && gate->stride(1) == 1, "gate must be [N, H] of q's dtype");
+    gstride = gate->stride(0);
+  }
+  ScalarExtras x;
+  if (sink_logits.has_value()) {
+    sk = f32c(*sink_logits);
+    TORCH_CHECK(sk.is_cuda() && sk.numel() == H, "sink_logits must be [H]");
+    x.sink_logits = sk.data_ptr<float>();
+  }
+  if (dist_bias.has_value()) {
+    db = f32c(*dist_bias);
+    TORCH_CHECK(db.is_cuda() && db.dim() == 2 && db.size(1) == H && db.size(0) >= 1, "dist_bias must be [rows, H]");
+    x.dist_bias = db.data_ptr<float>();
+    x.dist_rows = (int)db.size(0);
+  }
+  if (ksum.has_value()) {
+    TORCH_CHECK(vsum.has_value() && window > 0 && sum_block >= 1, "block summaries need both pools, a window and a block length");
+    const int rows = (int)ksum->size(1);
+    TORCH_CHECK(ksum->dim() == 4 && vsum->dim() == 4 && ksum->is_contiguous() && vsum->is_contiguous() &&
+                ksum->scalar_type() == q.scalar_type() && vsum->scalar_type() == q.scalar_type() &&
+                ksum->size(0) == kpool.size(0) && vsum->size(0) == kpool.size(0) && vsum->size(1) == rows &&
+                ksum->size(2) == G && ksum->size(3) == D && vsum->size(2) == G && vsum->size(3) == Dv &&
+                rows > 0 && (rows & (rows - 1)) == 0 && (long)rows * sum_block >= page,
+                "summary pools must be [pages, rows, G, D] / [.., Dv] of the pools' type, rows a power of two with "
+                "rows * block >= page size");
+    while ((1 << x.sum_shift) < rows) ++x.sum_shift;
+    x.sum_block = (int)sum_block;
+    x.ksum = ksum->data_ptr();
+    x.vsum = vsum->data_ptr();
+  }
+  at::Tensor out = cross ? at::empty({N, H, G, Dv}, q.options().dtype(at::kFloat)) : at::empty({N, H, Dv}, q.options());
+  if (N == 0) return out;
+  if (cross) x.cross_out = out.data_ptr<float>();
+  launch_scalar_attention(out, q, kpool, vpool, block_tables, tok_seq, positions, slp, gate, gstride, scale, window,
+                          keep_first, softcap, sink, page_shift, (long)vpool.stride(1), (long)vpool.stride(2), x);
+  return out;
+}
+
+// ------------------------------------------------------------------ block summaries
+// One wave per (sequence, block completed in this step, kv head): the float32 mean of the block's `block` cached
+// key rows and value rows goes to row b of the summary pools (page bt[b >> sum_shift], row b & mask).
+template <typename T>
+__global__ __launch_bounds__(64) void paged_pool_write_kernel(
+    T* __restrict__ ksum, T* __restrict__ vsum, const T* __restrict__ kpool, const T* __restrict__ vpool,
+    const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ cu, const int* __restrict__ start,
+    int G, int D, int Dv, int page_shift, int sum_shift, int block) {
+  const int b = blockIdx.x, g = blockIdx.z;
+  const int s0 = start[b], n = cu[b + 1] - cu[b];
+  const int blk = s0 / block + (int)blockIdx.y;
+  if (blk >= (s0 + n) / block) return;
+  const int* bt = block_tables + (long)b * bt_stride;
+  const int page_mask = (1 << page_shift) - 1, sum_mask = (1 << sum_shift) - 1;
+  const long srow = ((long)bt[blk >> sum_shift] << sum_shift) + (blk & sum_mask);
+  const float inv = 1.0f / (float)block;
+  for (int d = threadIdx.x; d < D + Dv; d += 64) {
+    const bool key = d < D;
+    float acc = 0.0f;
+    for (int i = 0; i < block; ++i) {
+      const int j = blk * block + i;
+      const long row = ((long)bt[j >> page_shift] << page_shift) + (j & page_mask);
+      acc += key ? ldf(kpool + (row * G + g) * D + d) : ldf(vpool + (row * G + g) * Dv + (d - D));
+    }
+    if (key) stf(ksum + (srow * G + g) * D + d, acc * inv);
+    else stf(vsum + (srow * G + g) * Dv + (d - D), acc * inv);
+  }
+}
+
+void paged_pool_write(at::Tensor kpool, at::Tensor vpool, at::Tensor ksum, at::Tensor vsum, at::Tensor block_tables,
+                      at::Tensor cu, at::Tensor start, int64_t block, int64_t most_blocks) {
+  check_act(kpool, "kpool");
+  TORCH_CHECK(kpool.dim() == 4 && vpool.dim() == 4 && ksum.dim() == 4 && vsum.dim() == 4 && kpool.is_contiguous() &&
+              vpool.is_contiguous() && ksum.is_contiguous() && vsum.is_contiguous(), "pools must be contiguous");
+  TORCH_CHECK(vpool.scalar_type() == kpool.scalar_type() && ksum.scalar_type() == kpool.scalar_type() &&
+              vsum.scalar_type() == kpool.scalar_type(), "pools share one dtype");
+  const int page = (int)kpool.size(1), G = (int)kpool.size(2), D = (int)kpool.size(3), Dv = (int)vpool.size(3);
+  const int rows = (int)ksum.size(1);
+  TORCH_CHECK(ksum.size(0) == kpool.size(0) && vsum.size(0) == kpool.size(0) && vsum.size(1) == rows &&
+              ksum.size(2) == G && ksum.size(3) == D && vsum.size(2) == G && vsum.size(3) == Dv && vpool.size(2) == G &&
+              vpool.size(1) == page, "summary pools do not fit the pools");
+  TORCH_CHECK(block >= 1 && rows > 0 && (rows & (rows - 1)) == 0 && (page & (page - 1)) == 0 &&
+              (long)rows * block >= page, "rows per page: a power of two with rows * block >= page size");
+  check_i32(block_tables, "block_tables"); check_i32(cu, "cu"); check_i32(start, "start");
+  const int B = (int)start.numel();
+  if (B == 0 || most_blocks <= 0) return;
+  int page_shift = 0, sum_shift = 0;
+  while ((1 << page_shift) < page) ++page_shift;
+  while ((1 << sum_shift) < rows) ++sum_shift;
+  SERVING_DISPATCH_ACT(kpool, T, {
+    hipLaunchKernelGGL(paged_pool_write_kernel<T>, dim3((unsigned)B, (unsigned)most_blocks, (unsigned)G), dim3(64), 0,
+                       stream(), ptr<T>(ksum), ptr<T>(vsum), ptr<T>(kpool), ptr<T>(vpool), block_tables.data_ptr<int>(),
+                       (int)block_tables.stride(0), cu.data_ptr<int>(), start.data_ptr<int>(), G, D, Dv, page_shift,
+                       sum_shift, (int)block);
+  });
+  HIP_CHECK_LAST();
 }
 
 }  // namespace serving
