@@ -190,3 +190,69 @@ def model_forward(config, tensors, tokens):
         residuals.append(x.clone())
     x = scalar_norm(x, tensors["final.norm"], eps)
     return x @ f64(tensors["head"]).T, residuals
+
+
+def forward(config, tensors, tokens):
+    return model_forward(config, tensors, tokens)[0]
+
+
+def random_checkpoint(config, seed=0, rel_rows=10):
+    """Random tensors for a config, named and shaped as a checkpoint holds them (bfloat16)."""
+    g = torch.Generator().manual_seed(seed)
+    W = config["width"]
+    out = {}
+
+    def put(name, *shape, std=1.0, mean=0.0):
+        out[name] = (torch.randn(shape, generator=g) * std + mean).to(torch.bfloat16)
+
+    def attention(pre, c, extra):
+        H, G, D, Dv = c["heads"], c["kv_heads"], c["dim"], c["vdim"]
+        for n, rows in (("q", H * D), ("k", G * D), ("v", G * Dv)):
+            put(pre + n, rows, W, std=W ** -0.5)
+            put(pre + n + ".b", rows, std=0.3)
+        put(pre + "o", W, H * Dv, std=(H * Dv) ** -0.5)
+        put(pre + "o.b", W, std=0.3)
+        extra(H)
+
+    def expert(pre, ff):
+        put(pre + "gate", ff, W, std=W ** -0.5)
+        put(pre + "up", ff, W, std=W ** -0.5)
+        put(pre + "down", W, ff, std=ff ** -0.5)
+
+    put("embed", config["vocab"], W)
+    put("head", config["vocab"], W, std=W ** -0.5)
+    put("final.norm", std=0.1, mean=1.2)
+    for i, spec in enumerate(config["layers"]):
+        pre, m = f"l{i}.", spec["mixer"]
+        put(pre + "norm1", std=0.1, mean=0.8)
+        if spec["type"] == "attention":
+            def extra(H, pre=pre):
+                put(pre + "mix.rel", rel_rows, H)
+                put(pre + "mix.sink", H)
+                put(pre + "mix.vmix", std=0.05, mean=0.35)
+            attention(pre + "mix.", m, extra)
+        else:
+            def extra(H, pre=pre):
+                out[pre + "mix.left.talk"] = (torch.eye(H) + 0.3 * torch.randn(H, H, generator=g)).to(torch.bfloat16)
+            attention(pre + "mix.left.", m["left"], extra)
+            r, q = m["right"], pre + "mix.right."
+            put(q + "in", 2 * r["inner"], W, std=W ** -0.5)
+            put(q + "conv", r["inner"], r["conv"], std=0.5)
+            put(q + "conv.b", r["inner"], std=0.2)
+            put(q + "x", r["dt_rank"] + 2 * r["state"], r["inner"], std=r["inner"] ** -0.5)
+            put(q + "dt", r["inner"], r["dt_rank"], std=r["dt_rank"] ** -0.5)
+            put(q + "dt.b", r["inner"], std=0.5)
+            put(q + "A_log", r["inner"], r["state"], std=0.5)
+            put(q + "D", r["inner"])
+            put(q + "o", W, r["inner"], std=r["inner"] ** -0.5)
+        f = spec.get("mlp")
+        if f is not None:
+            put(pre + "norm2", std=0.1, mean=0.9)
+            E, I = f["router"]["experts"], f["router"].get("identity", 0)
+            put(pre + "mlp.router", E + I, W, std=2.0 * W ** -0.5)
+            put(pre + "mlp.correction", E + I, std=0.05)
+            for e in range(E):
+                expert(pre + f"mlp.e{e}.", f["expert"]["ff"])
+            if f.get("shared"):
+                expert(pre + "mlp.shared.", f["shared"]["ff"])
+    return out
