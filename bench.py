@@ -29,11 +29,12 @@ def parse_args():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=5)
     p.add_argument("--warmup", type=int, default=2)
-    p.add_argument("--workload", type=str, default="train", choices=["train", "serve-hybrid", "serve-moe", "serve-latent"],
-                   help="train: the headline training step (default). serve-hybrid / serve-moe / serve-latent: "
-                        "prefill/decode tokens/s of the Kipirax hybrid / the Mubutar routed-experts model / the Vitinex "
-                        "latent-attention + state-space model next to a Llama of equal size (Vitinex also next to "
-                        "Mubutar), all through the continuous-batching engine")
+    p.add_argument("--workload", type=str, default="train", choices=["train", "serve-hybrid", "serve-moe", "serve-latent", "serve-pooled"],
+                   help="train: the headline training step (default). serve-hybrid / serve-moe / serve-latent / "
+                        "serve-pooled: prefill/decode tokens/s of the Kipirax hybrid / the Mubutar routed-experts model / "
+                        "the Vitinex latent-attention + state-space model / the Tarulix window + block-summary + "
+                        "selective-scan model next to a Llama of equal size (the last two also next to Mubutar), all "
+                        "through the continuous-batching engine")
     p.add_argument("--serve-sizes", type=str, default="w2048,w4096")
     p.add_argument("--model", type=str, default="llama-7b")
     p.add_argument("--batch", type=int, default=36, help="per-DP-rank batch size (reference: bs/DP=36)")
@@ -69,7 +70,7 @@ def serve_comparison(args, kind):
 
 def main():
     args = parse_args()
-    if args.workload in ("serve-hybrid", "serve-moe", "serve-latent"):
+    if args.workload in ("serve-hybrid", "serve-moe", "serve-latent", "serve-pooled"):
         return serve_comparison(args, args.workload.split("-")[1])
     import colossalai_amd
     from colossalai_amd.models import LLAMA_CONFIGS, LlamaForCausalLM, llama_flops_per_token

@@ -21,12 +21,13 @@ at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at:
                            at::Tensor start, at::Tensor tok_seq, at::Tensor positions, double scale, int64_t window,
                            int64_t keep_first, c10::optional<at::Tensor> slopes, c10::optional<at::Tensor> gate,
                            int64_t num_tiles, double softcap, bool sink, int64_t num_tiles128);
-at::Tensor paged_attention_ext(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at::Tensor block_tables,
-                               at::Tensor tok_seq, at::Tensor positions, double scale, int64_t window,
+at::Tensor paged_attention_ext(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at::Tensor block_tables, at::Tensor cu,
+                               at::Tensor start, at::Tensor tok_seq, at::Tensor positions, double scale, int64_t window,
                                int64_t keep_first, c10::optional<at::Tensor> slopes, c10::optional<at::Tensor> gate,
                                double softcap, bool sink, c10::optional<at::Tensor> sink_logits,
                                c10::optional<at::Tensor> dist_bias, c10::optional<at::Tensor> ksum,
-                               c10::optional<at::Tensor> vsum, int64_t sum_block, bool cross);
+                               c10::optional<at::Tensor> vsum, int64_t sum_block, bool cross, int64_t num_tiles,
+                               int64_t num_tiles128);
 void paged_pool_write(at::Tensor kpool, at::Tensor vpool, at::Tensor ksum, at::Tensor vsum, at::Tensor block_tables,
                       at::Tensor cu, at::Tensor start, int64_t block, int64_t most_blocks);
 at::Tensor rotate_halves_unit_norm(at::Tensor x, at::Tensor positions, c10::optional<at::Tensor> freqs, double eps,

@@ -302,7 +302,14 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     const bf16s* __restrict__ vpool, const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ cu,
     const int* __restrict__ start, const float* __restrict__ slopes, const bf16s* __restrict__ gate, long gate_stride,
     int H, int G, int Dr, int Dvr, int page_shift, float scale, int window, int keep_first, float softcap, int sink,
-    int qsplit) {
+    int qsplit, const float* __restrict__ sink2, const float* __restrict__ dist2, int dist_rows,
+    const bf16s* __restrict__ ksum, const bf16s* __restrict__ vsum, int sum_shift, int sum_block,
+    float* __restrict__ cross_out) {
+  // The optional extras of the split-key kernel, in the base-2 domain: sink2 [H] = learned sink scores * log2e;
+  // dist2 [H, dist_rows] = the per-distance bias * log2e, one row per head; ksum / vsum = block summaries, staged as
+  // the first tiles of a block (summary idx of a sequence is seen by a token at pos when idx < (pos - window + 1) /
+  // sum_block); cross_out [N, H, G, Dv] float32: the grid's z axis then also counts the kv head whose values a block
+  // multiplies the weights with.
   // qsplit (kv heads with a single query head each): the four waves of a block are four consecutive 32-token tiles
   // of that head instead of four heads, so a block covers 128 tokens, the grid's x axis counts 128-token tiles, and
   // the staged key/value tiles are still shared by all computing waves. The block stages the key range of all its
@@ -321,7 +328,9 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   const int tid = threadIdx.x;
   const int wid = tid >> 6, lane = tid & 63;
   const int rep = H / G, g = blockIdx.y;
-  const int hl = qsplit ? 0 : blockIdx.z * (nthreads >> 6) + wid;  // head inside the group
+  const int VC = cross_out != nullptr ? G : 1;
+  const int vg = cross_out != nullptr ? (int)(blockIdx.z % VC) : g;   // kv head of the values
+  const int hl = qsplit ? 0 : (blockIdx.z / VC) * (nthreads >> 6) + wid;  // head inside the group
   const int h = g * rep + (hl < rep ? hl : 0);
   const int bshift = qsplit ? 7 : 5;                  // log2 of the tokens a block covers
   // Under a causal mask a late tile of a long prompt has many more key tiles than an early one. Rows of the grid
@@ -359,8 +368,13 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   const int lo_min = window > 0 ? max(0, bp0 - window + 1) : 0;   // the staged key range is the block's
   const int wstart = lo_min & ~31;
   const int n_sink = window > 0 ? min(keep_first, wstart) : 0;  // kept keys below the window's first tile
-  const int sink_tiles = (n_sink + 31) >> 5;
+  const int n_sum = (ksum != nullptr && window > 0) ? max(0, (bp1 - window + 1) / sum_block) : 0;  // the block's last token's
+  const int sum_tiles = (n_sum + 31) >> 5;
+  const int sum_mask = (1 << sum_shift) - 1;
+  const int sink_tiles = sum_tiles + ((n_sink + 31) >> 5);   // summary tiles, then kept-prefix tiles, then the window's
   const int tiles_n = sink_tiles + ((bp1 - wstart) >> 5) + 1;
+  const int my_sum = (ksum != nullptr && window > 0) ? max(0, (pos - window + 1) / sum_block) : 0;  // this token's
+  const float* db = dist2 != nullptr ? dist2 + (long)h * dist_rows : nullptr;
 
   // staging: key chunk c = key c / (row chunks), 8 elements starting at 8 * (c % row chunks), stored as a row;
   // value chunk c = key c % 32, 8 channels starting at 8 * (c / 32): the values are stored transposed, two bytes at
@@ -369,39 +383,51 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   // TP key tiles are staged, and multiplied, between two barriers: their loads are all in flight over the
   // products of the TP tiles before them
   bf16x8_v rk[TP][KR], rv[TP][VR];
-  auto tile_base = [&](int it) { return it < sink_tiles ? it * 32 : wstart + (it - sink_tiles) * 32; };
+  auto tile_base = [&](int it) {
+    return it < sum_tiles ? it * 32 : it < sink_tiles ? (it - sum_tiles) * 32 : wstart + (it - sink_tiles) * 32;
+  };
   auto pool_row = [&](int j) {
     const int jc = min(j, bp1);  // keys past the sequence's end are masked; read a row that exists
     return ((long)bt[jc >> page_shift] << page_shift) + (jc & page_mask);
   };
+  auto sum_row = [&](int idx) {
+    const int ic = min(idx, n_sum - 1);  // a summary tile exists only when n_sum > 0
+    return ((long)bt[ic >> sum_shift] << sum_shift) + (ic & sum_mask);
+  };
   // The page-table lookups of a tile run one tile ahead of its key/value loads (two ahead of its use), so that a
   // load's address never waits for a lookup issued in the same iteration.
   int krow[TP][KR], vrow[TP][VR];
+  bool from_sum[TP];  // the tiles of the last lookup that are summary tiles
   auto lookup = [&](int step) {
 #pragma unroll
     for (int u = 0; u < TP; ++u) {
       const int kbase = tile_base(step * TP + u);  // a tile past the last one reads rows that exist and is not used
+      from_sum[u] = step * TP + u < sum_tiles;
 #pragma unroll
       for (int r = 0; r < KR; ++r) {
         const int c = tid + nthreads * r;
-        krow[u][r] = c < KCH ? (int)pool_row(kbase + c / (D / 8)) : 0;
+        const int j = kbase + c / (D / 8);
+        krow[u][r] = c < KCH ? (int)(from_sum[u] ? sum_row(j) : pool_row(j)) : 0;
       }
 #pragma unroll
       for (int r = 0; r < VR; ++r) {
         const int c = tid + nthreads * r;
-        vrow[u][r] = c < VCH ? (int)pool_row(kbase + (c & 31)) : 0;
+        const int j = kbase + (c & 31);
+        vrow[u][r] = c < VCH ? (int)(from_sum[u] ? sum_row(j) : pool_row(j)) : 0;
       }
     }
   };
   auto fetch = [&]() {  // the tiles whose rows the last lookup left in krow / vrow
 #pragma unroll
     for (int u = 0; u < TP; ++u) {
+      const bf16s* kp = from_sum[u] ? ksum : kpool;
+      const bf16s* vp = from_sum[u] ? vsum : vpool;
 #pragma unroll
       for (int r = 0; r < KR; ++r) {
         const int c = tid + nthreads * r;
         if (c < KCH) {
           const int off = 8 * (c % (D / 8));
-          rk[u][r] = off < Dr ? ld_g16b(kpool + ((long)krow[u][r] * G + g) * Dr + off) : zero8;
+          rk[u][r] = off < Dr ? ld_g16b(kp + ((long)krow[u][r] * G + g) * Dr + off) : zero8;
         }
       }
 #pragma unroll
@@ -409,7 +435,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
         const int c = tid + nthreads * r;
         if (c < VCH) {
           const int off = 8 * (c >> 5);
-          rv[u][r] = off < Dvr ? ld_g16b(vpool + ((long)vrow[u][r] * G + g) * Dvr + off) : zero8;
+          rv[u][r] = off < Dvr ? ld_g16b(vp + ((long)vrow[u][r] * G + vg) * Dvr + off) : zero8;
         }
       }
     }
@@ -484,7 +510,8 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     for (int u = 0; u < TP; ++u) {
       const int it = step * TP + u;
       if (!head_ok || it >= tiles_n) continue;
-      const bool sink = it < sink_tiles;
+      const bool summ = it < sum_tiles;
+      const bool sink = it < sink_tiles;  // a tile ahead of the window's: summaries or kept first tokens
       const int kbase = tile_base(it);
       if (!sink && kbase > p1) continue;  // (query split) a tile wholly after this wave's tokens
       const int klimit = sink ? n_sink : p1 + 1;  // keys of this tile at or above it are not this tile's to count
@@ -503,7 +530,13 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
       const float tile_bias = -sl2 * (float)(pos - kbase);
       // interior tile: every key is visible to every token of the tile, no masks to evaluate
       const bool interior = !sink && t_off + 31 < cnt && kbase + 31 <= p0 && (window == 0 || p1 - kbase < window);
-      if (interior) {
+      if (summ) {  // summaries: seen by count, no distance terms
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int j = kbase + (i & 3) + 8 * (i >> 2) + 4 * hf;
+          sv[i] = (tok_ok && j < my_sum) ? base2(sacc[i]) : -INFINITY;
+        }
+      } else if (interior) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           sv[i] = base2(sacc[i]) + (tile_bias + row_bias[i]);
@@ -514,6 +547,13 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
           const int j = kbase + (i & 3) + 8 * (i >> 2) + 4 * hf;
           const bool seen = tok_ok && j < klimit && j <= pos && (window == 0 || pos - j < window || j < keep_first);
           sv[i] = seen ? base2(sacc[i]) + (tile_bias + row_bias[i]) : -INFINITY;
+        }
+      }
+      if (db != nullptr && !summ) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int j = kbase + (i & 3) + 8 * (i >> 2) + 4 * hf;
+          sv[i] += db[min(max(pos - j, 0), dist_rows - 1)];   // -inf stays -inf
         }
       }
       float m_ref = 0.0f, corr = 1.0f;
@@ -558,10 +598,24 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     __syncthreads();
   }
   l += __shfl_xor(l, 32);
-  if (sink) l += __builtin_amdgcn_exp2f(-m);  // the sink's score is 0 in either base; m is finite (a token sees itself)
+  if (sink2 != nullptr) l += __builtin_amdgcn_exp2f(sink2[h] - m);  // a learned score; a sink far above every key: 1 / inf = 0
+  else if (sink) l += __builtin_amdgcn_exp2f(-m);  // the sink's score is 0 in either base; m is finite (a token sees itself)
   if (!tok_ok || !head_ok) return;
   float scale_out = 1.0f / l;
   if (gate != nullptr) scale_out *= sigmoidf_(ldf(gate + n * gate_stride + h));
+  if (cross_out != nullptr) {
+    float* crow = cross_out + ((n * H + h) * G + vg) * (long)Dvr;
+#pragma unroll
+    for (int t = 0; t < VT; ++t)
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        if (t * 32 + 8 * a + 4 * hf >= Dvr) continue;
+        *reinterpret_cast<float4v*>(crow + t * 32 + 8 * a + 4 * hf) =
+            float4v{oacc[t][4 * a] * scale_out, oacc[t][4 * a + 1] * scale_out, oacc[t][4 * a + 2] * scale_out,
+                    oacc[t][4 * a + 3] * scale_out};
+      }
+    return;
+  }
   bf16s* orow = out + (n * H + h) * (long)Dvr;
 #pragma unroll
   for (int t = 0; t < VT; ++t)
@@ -635,6 +689,62 @@ static void launch_scalar_attention(at::Tensor& out, const at::Tensor& q, const 
   HIP_CHECK_LAST();
 }
 
+// The matrix-core kernel for prompt portions in bfloat16 whose head sizes fit a tiling; false when it does not apply.
+// In `x`, sink_logits and dist_bias are already in the base-2 domain (times log2 e), dist_bias one row per head.
+static bool launch_mfma_attention(at::Tensor& out, const at::Tensor& q, const at::Tensor& kpool, const at::Tensor& vpool,
+                                  const at::Tensor& block_tables, const at::Tensor& cu, const at::Tensor& start,
+                                  const float* slp, const c10::optional<at::Tensor>& gate, long gstride, double scale,
+                                  int64_t window, int64_t keep_first, double softcap, bool sink, int page_shift,
+                                  int64_t num_tiles, int64_t num_tiles128, const ScalarExtras& x) {
+  const int H = (int)q.size(1), D = (int)q.size(2);
+  const int G = (int)kpool.size(2), Dv = (int)vpool.size(3);
+  // prompt portions in bfloat16 go to the matrix cores when the head sizes fit a tiling;
+  // num_tiles = sum over sequences of ceil(new tokens / 32), 0 asks for the scalar kernel
+  const bool aligned = q.stride(0) % 8 == 0 && reinterpret_cast<uintptr_t>(q.data_ptr()) % 16 == 0;
+  // head sizes that are multiples of 8 ride in the next larger tiling, zero-padded
+  const bool mfma_shape = D % 8 == 0 && Dv % 8 == 0 && D <= 128 && Dv <= 128;
+  if (!(num_tiles > 0 && is_bf16(q) && aligned && mfma_shape && vpool.is_contiguous())) return false;
+  {
+    const int rep = H / G, nw = 4;
+    // one query head per kv head: the waves of a block take four consecutive token tiles instead of four heads
+    const int qsplit = (rep == 1 && num_tiles128 > 0) ? 1 : 0;
+    const int VC = x.cross_out != nullptr ? G : 1;
+    const dim3 grid((unsigned)(qsplit ? num_tiles128 : num_tiles), (unsigned)G, (unsigned)((rep + nw - 1) / nw * VC));
+    const int ds = D <= 32 ? 2 : D <= 48 ? 3 : D <= 64 ? 4 : D <= 96 ? 6 : 8, vt = (Dv + 31) / 32;
+    const size_t msmem = (size_t)2 * MFMA_TILES_PER_STEP * (32 * (ds * 16 + 8) + vt * 32 * 40) * sizeof(bf16s);
+#define MFMA_CASE(DS_, VT_)                                                                                        \
+  do {                                                                                                             \
+    auto kfn = paged_attention_mfma_kernel<DS_, VT_>;                                                              \
+    if (msmem > 65536) /* more dynamic LDS than a kernel gets without asking */                                    \
+      (void)hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)msmem);         \
+    hipLaunchKernelGGL(kfn, grid, dim3(64 * nw), msmem, stream(),                                                 \
+                       x.cross_out != nullptr ? (bf16s*)nullptr : ptr<bf16s>(out), ptr<bf16s>(q),                  \
+                       (long)q.stride(0), ptr<bf16s>(kpool), ptr<bf16s>(vpool), block_tables.data_ptr<int>(),      \
+                       (int)block_tables.stride(0), cu.data_ptr<int>(), start.data_ptr<int>(), slp,                \
+                       gate.has_value() ? ptr<bf16s>(*gate) : (const bf16s*)nullptr, gstride, H, G, D, Dv,         \
+                       page_shift, (float)scale, (int)window, (int)keep_first, (float)softcap, sink ? 1 : 0,       \
+                       qsplit, x.sink_logits, x.dist_bias, x.dist_rows, (const bf16s*)x.ksum,                      \
+                       (const bf16s*)x.vsum, x.sum_shift, x.sum_block, x.cross_out);                               \
+  } while (0)
+#define MFMA_ROW(DS_)                     \
+  do {                                    \
+    if (vt == 1) MFMA_CASE(DS_, 1);       \
+    else if (vt == 2) MFMA_CASE(DS_, 2);  \
+    else if (vt == 3) MFMA_CASE(DS_, 3);  \
+    else MFMA_CASE(DS_, 4);               \
+  } while (0)
+    if (ds == 2) MFMA_ROW(2);
+    else if (ds == 3) MFMA_ROW(3);
+    else if (ds == 4) MFMA_ROW(4);
+    else if (ds == 6) MFMA_ROW(6);
+    else MFMA_ROW(8);
+#undef MFMA_ROW
+#undef MFMA_CASE
+    HIP_CHECK_LAST();
+    return true;
+  }
+}
+
 at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at::Tensor block_tables, at::Tensor cu,
                            at::Tensor start, at::Tensor tok_seq, at::Tensor positions, double scale, int64_t window,
                            int64_t keep_first, c10::optional<at::Tensor> slopes, c10::optional<at::Tensor> gate,
@@ -675,47 +785,9 @@ at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at:
   at::Tensor out = at::empty({N, H, Dv}, q.options());
   if (N == 0) return out;
   check_i32(cu, "cu"); check_i32(start, "start");
-  // prompt portions in bfloat16 go to the matrix cores when the head sizes fit a tiling;
-  // num_tiles = sum over sequences of ceil(new tokens / 32), 0 asks for the scalar kernel
-  const bool aligned = q.stride(0) % 8 == 0 && reinterpret_cast<uintptr_t>(q.data_ptr()) % 16 == 0;
-  // head sizes that are multiples of 8 ride in the next larger tiling, zero-padded
-  const bool mfma_shape = D % 8 == 0 && Dv % 8 == 0 && D <= 128 && Dv <= 128;
-  if (num_tiles > 0 && is_bf16(q) && aligned && mfma_shape && vpool.is_contiguous()) {
-    const int rep = H / G, nw = 4;
-    // one query head per kv head: the waves of a block take four consecutive token tiles instead of four heads
-    const int qsplit = (rep == 1 && num_tiles128 > 0) ? 1 : 0;
-    const dim3 grid((unsigned)(qsplit ? num_tiles128 : num_tiles), (unsigned)G, (unsigned)((rep + nw - 1) / nw));
-    const int ds = D <= 32 ? 2 : D <= 48 ? 3 : D <= 64 ? 4 : D <= 96 ? 6 : 8, vt = (Dv + 31) / 32;
-    const size_t msmem = (size_t)2 * MFMA_TILES_PER_STEP * (32 * (ds * 16 + 8) + vt * 32 * 40) * sizeof(bf16s);
-#define MFMA_CASE(DS_, VT_)                                                                                        \
-  do {                                                                                                             \
-    auto kfn = paged_attention_mfma_kernel<DS_, VT_>;                                                              \
-    if (msmem > 65536) /* more dynamic LDS than a kernel gets without asking */                                    \
-      (void)hipFuncSetAttribute((const void*)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)msmem);         \
-    hipLaunchKernelGGL(kfn, grid, dim3(64 * nw), msmem, stream(), ptr<bf16s>(out), ptr<bf16s>(q),                  \
-                       (long)q.stride(0), ptr<bf16s>(kpool), ptr<bf16s>(vpool), block_tables.data_ptr<int>(),      \
-                       (int)block_tables.stride(0), cu.data_ptr<int>(), start.data_ptr<int>(), slp,                \
-                       gate.has_value() ? ptr<bf16s>(*gate) : (const bf16s*)nullptr, gstride, H, G, D, Dv,         \
-                       page_shift, (float)scale, (int)window, (int)keep_first, (float)softcap, sink ? 1 : 0,       \
-                       qsplit);                                                                                    \
-  } while (0)
-#define MFMA_ROW(DS_)                     \
-  do {                                    \
-    if (vt == 1) MFMA_CASE(DS_, 1);       \
-    else if (vt == 2) MFMA_CASE(DS_, 2);  \
-    else if (vt == 3) MFMA_CASE(DS_, 3);  \
-    else MFMA_CASE(DS_, 4);               \
-  } while (0)
-    if (ds == 2) MFMA_ROW(2);
-    else if (ds == 3) MFMA_ROW(3);
-    else if (ds == 4) MFMA_ROW(4);
-    else if (ds == 6) MFMA_ROW(6);
-    else MFMA_ROW(8);
-#undef MFMA_ROW
-#undef MFMA_CASE
-    HIP_CHECK_LAST();
+  if (launch_mfma_attention(out, q, kpool, vpool, block_tables, cu, start, slp, gate, gstride, scale, window, keep_first,
+                            softcap, sink, page_shift, num_tiles, num_tiles128, ScalarExtras()))
     return out;
-  }
   launch_scalar_attention(out, q, kpool, vpool, block_tables, tok_seq, positions, slp, gate, gstride, scale, window,
                           keep_first, softcap, sink, page_shift, vrow, vhead, ScalarExtras());
   return out;
@@ -724,12 +796,13 @@ at::Tensor paged_attention(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at:
 // The split-key kernel with its optional extras, for prompt portions and decode tokens alike: a learned sink per
 // head, a per-distance bias table, block summaries ahead of the window, and (cross) every query head's weights
 // applied to every kv head's values, returned as float32 [N, H, G, Dv] for a talking-heads mix.
-at::Tensor paged_attention_ext(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at::Tensor block_tables,
-                               at::Tensor tok_seq, at::Tensor positions, double scale, int64_t window,
+at::Tensor paged_attention_ext(at::Tensor q, at::Tensor kpool, at::Tensor vpool, at::Tensor block_tables, at::Tensor cu,
+                               at::Tensor start, at::Tensor tok_seq, at::Tensor positions, double scale, int64_t window,
                                int64_t keep_first, c10::optional<at::Tensor> slopes, c10::optional<at::Tensor> gate,
                                double softcap, bool sink, c10::optional<at::Tensor> sink_logits,
                                c10::optional<at::Tensor> dist_bias, c10::optional<at::Tensor> ksum,
-                               c10::optional<at::Tensor> vsum, int64_t sum_block, bool cross) {
+                               c10::optional<at::Tensor> vsum, int64_t sum_block, bool cross, int64_t num_tiles,
+                               int64_t num_tiles128) {
   check_act(q, "q");
   TORCH_CHECK(softcap >= 0.0, "softcap must not be negative (0 = none)");
   TORCH_CHECK(q.dim() == 3 && q.stride(2) == 1 && q.stride(1) == q.size(2), "q must be [N, H, D] with dense rows");
@@ -790,6 +863,23 @@ at::Tensor paged_attention_ext(at::Tensor q, at::Tensor kpool, at::Tensor vpool,
   at::Tensor out = cross ? at::empty({N, H, G, Dv}, q.options().dtype(at::kFloat)) : at::empty({N, H, Dv}, q.options());
   if (N == 0) return out;
   if (cross) x.cross_out = out.data_ptr<float>();
+  if (num_tiles > 0 && is_bf16(q)) {  // prompt portions in bfloat16: the matrix-core kernel, extras in the base-2 domain
+    check_i32(cu, "cu"); check_i32(start, "start");
+    constexpr double LOG2E = 1.4426950408889634;
+    ScalarExtras x2 = x;
+    at::Tensor sk2, db2;
+    if (sink_logits.has_value()) {
+      sk2 = sk * LOG2E;
+      x2.sink_logits = sk2.data_ptr<float>();
+    }
+    if (dist_bias.has_value()) {
+      db2 = (db * LOG2E).t().contiguous();   // [H, rows]
+      x2.dist_bias = db2.data_ptr<float>();
+    }
+    if (launch_mfma_attention(out, q, kpool, vpool, block_tables, cu, start, slp, gate, gstride, scale, window,
+                              keep_first, softcap, sink, page_shift, num_tiles, num_tiles128, x2))
+      return out;
+  }
   launch_scalar_attention(out, q, kpool, vpool, block_tables, tok_seq, positions, slp, gate, gstride, scale, window,
                           keep_first, softcap, sink, page_shift, (long)vpool.stride(1), (long)vpool.stride(2), x);
   return out;

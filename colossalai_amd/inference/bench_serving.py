@@ -1,11 +1,13 @@
 """Serving throughput of the ragged-step models next to a Llama of equal width,
 depth and per-token work, all through ``ContinuousBatchEngine``: prefill tokens/s
 of one long prompt and decode tokens/s of a batch of running sequences. Random
-weights, synthetic tokens. Three comparisons: the Kipirax hybrid (paged window
+weights, synthetic tokens. Four comparisons: the Kipirax hybrid (paged window
 attention + recurrent state), Mubutar (sink-softmax attention with shared
-keys, routed experts) and Vitinex (latent attention + state-space layers in a
-looped block, routed experts), the last also next to Mubutar, whose kernels are
-the closest.
+keys, routed experts), Vitinex (latent attention + state-space layers in a
+looped block, routed experts) and Tarulix (windowed attention with a distance
+table and a learned sink; window + block summaries + talking heads beside a
+selective scan; gated experts with identity experts), the last two also next to
+Mubutar, whose kernels are the closest.
 """
 
 import json
@@ -15,11 +17,12 @@ from typing import Dict, List
 import torch
 
 from ..models import (KipiraxConfig, KipiraxForCausalLM, LlamaConfig, LlamaForCausalLM, MubutarConfig,
-                      MubutarForCausalLM, VitinexConfig, VitinexForCausalLM)
+                      MubutarForCausalLM, TarulixConfig, TarulixForCausalLM, VitinexConfig, VitinexForCausalLM)
 from .config import InferenceConfig
 from .paged_engine import ContinuousBatchEngine
 
-__all__ = ["SIZES", "hybrid_config", "llama_config", "moe_config", "latent_config", "run_serving_comparison"]
+__all__ = ["SIZES", "hybrid_config", "llama_config", "moe_config", "latent_config", "pooled_config",
+           "run_serving_comparison"]
 
 # width, layers, heads, kv_heads, head size, vocab
 SIZES = {
@@ -90,6 +93,26 @@ def latent_config(s: dict, experts: int = 32, top: int = 6) -> VitinexConfig:
                          loop=dict(start=0, stop=2, times=2))
 
 
+def pooled_config(s: dict, experts: int = 32, top: int = 6, window: int = 1024, pool: int = 64) -> TarulixConfig:
+    """Windowed attention (distance table of 32 rows, learned sink, values mixed with the first layer's) and the
+    parallel mixer (window + summaries of 64 positions + talking heads beside a selective scan of twice the width
+    inside, 16 state places, 4 taps) in turn, Llama's head sizes; every layer carries routed gated experts of
+    Mubutar's sizes (three matrices each, so two thirds of its hidden width) plus two identity experts."""
+    W, H, G, D = s["width"], s["heads"], s["kv_heads"], s["dim"]
+    inter = _inter(W)
+    ff = W // 3 // 32 * 32
+    shared = (inter - top * ff + 127) // 128 * 128
+    att = dict(bias_max=float(window), dim=D, heads=H, kv_heads=G, vdim=D, scale=1.0, mask=dict(size=window), v_mix=True)
+    left = dict(dim=D, heads=H, kv_heads=G, vdim=D, scale=1.0, softcap=30.0, mask=dict(size=window, pool=pool),
+                rot=dict(base=250000.0, dims=D // 2))
+    right = dict(conv=4, dt_rank=W // 16, inner=2 * W, state=16)
+    mlp = dict(kind="moe", expert=dict(ff=ff), shared=dict(ff=shared), router=dict(experts=experts, identity=2, top=top))
+    layers = [dict(type="attention", mixer=att, mlp=mlp) if i % 2 == 0 else
+              dict(type="parallel", mixer=dict(left=left, right=right, left_scale=0.8, right_scale=0.5), mlp=mlp)
+              for i in range(s["layers"])]
+    return TarulixConfig(vocab=s["vocab"], width=W, layers=layers, norm_eps=1e-6)
+
+
 def llama_config(s: dict, max_positions: int) -> LlamaConfig:
     # gate/up/down of 8/3 W carry the parameters of the hybrid's up/down of 4 W
     inter = _inter(s["width"])
@@ -151,6 +174,24 @@ def _latent_numbers(s: dict, prompt: int, batch: int, context: int, steps: int) 
     return _ragged_numbers(model, cfg.vocab, prompt, batch, context, steps)
 
 
+def _pooled_numbers(s: dict, prompt: int, batch: int, context: int, steps: int) -> Dict[str, float]:
+    cfg = pooled_config(s)
+    model = _random(TarulixForCausalLM(cfg), torch.bfloat16)
+    with torch.no_grad():
+        for layer in model.layers:     # what enters scores, routers and the recurrence stays float32
+            layer.mlp.router.data = layer.mlp.router.data.float()
+            for att in ([layer.mix] if layer.kind == "attention" else [layer.mix.left]):
+                att.in_proj.bias.data = att.in_proj.bias.data.to(torch.bfloat16)
+                att.o.bias.data = att.o.bias.data.to(torch.bfloat16)
+            if layer.kind == "attention":
+                layer.mix.rel.data = layer.mix.rel.data.float()
+            else:
+                layer.mix.left.talk.data = torch.eye(layer.mix.left.H, device="cuda") + layer.mix.left.talk.data.float()
+                layer.mix.right.conv.data = layer.mix.right.conv.data.float().normal_(0, 0.3)
+                layer.mix.right.A_log.data = layer.mix.right.A_log.data.float()
+    return _ragged_numbers(model, cfg.vocab, prompt, batch, context, steps)
+
+
 def _ragged_numbers(model, vocab: int, prompt: int, batch: int, context: int, steps: int) -> Dict[str, float]:
     page = 64
     blocks = max(prompt, batch * (context + steps + page)) // page + batch + 2
@@ -206,14 +247,14 @@ def _llama_numbers(s: dict, prompt: int, batch: int, context: int, steps: int) -
 
 def run_serving_comparison(sizes: List[str], prompt: int = 4096, batch: int = 16, context: int = 1024,
                            steps: int = 32, kind: str = "hybrid") -> dict:
-    """``kind``: "hybrid" (Kipirax), "moe" (Mubutar) or "latent" (Vitinex), each next to Llama; "latent" also
-    next to Mubutar."""
-    ours = {"hybrid": _hybrid_numbers, "moe": _moe_numbers, "latent": _latent_numbers}[kind]
+    """``kind``: "hybrid" (Kipirax), "moe" (Mubutar), "latent" (Vitinex) or "pooled" (Tarulix), each next to
+    Llama; "latent" and "pooled" also next to Mubutar."""
+    ours = {"hybrid": _hybrid_numbers, "moe": _moe_numbers, "latent": _latent_numbers, "pooled": _pooled_numbers}[kind]
     out = {}
     for name in sizes:
         s = SIZES[name]
         out[name] = {kind: ours(s, prompt, batch, context, steps)}
-        if kind == "latent":
+        if kind in ("latent", "pooled"):
             out[name]["moe"] = _moe_numbers(s, prompt, batch, context, steps)
         out[name]["llama"] = _llama_numbers(s, prompt, batch, context, steps)
         out[name]["shape"] = dict(s, prompt=prompt, batch=batch, context=context)

@@ -194,13 +194,13 @@ def paged_attention(q, kpool, vpool, batch: RaggedBatch, scale: float, window: i
     (key summaries, value summaries, block) needs a window; ``talk`` [H, H]."""
     assert pooled is None or window > 0, "block summaries stand for what a window no longer shows"
     if use_hip(q) and (sink_logits is not None or dist_bias is not None or pooled is not None or talk is not None):
-        # these run on the split-key kernel for prompt portions too. With talking heads it hands back every query
-        # head's weights applied to every key/value head's values, O[n, g, c] (float32): the mix is linear, so
-        # out[n, h] = sum_g talk[h, g] O[n, g, kv(h)]
+        # With talking heads the kernels hand back every query head's weights applied to every key/value head's
+        # values, O[n, g, c] (float32): the mix is linear, so out[n, h] = sum_g talk[h, g] O[n, g, kv(h)]
         ksum, vsum, block = pooled if pooled is not None else (None, None, 0)
-        o = serving_kernels().paged_attention_ext(q, kpool, vpool, batch.block_tables, batch.tok_seq, batch.positions,
-                                                  scale, window, keep_first, slopes, gate, float(softcap), bool(sink),
-                                                  sink_logits, dist_bias, ksum, vsum, int(block), talk is not None)
+        o = serving_kernels().paged_attention_ext(q, kpool, vpool, batch.block_tables, batch.cu, batch.start,
+                                                  batch.tok_seq, batch.positions, scale, window, keep_first, slopes,
+                                                  gate, float(softcap), bool(sink), sink_logits, dist_bias, ksum, vsum,
+                                                  int(block), talk is not None, batch.num_tiles32, batch.num_tiles128)
         if talk is None:
             return o
         return serving_kernels().talk_mix(o, talk, q.dtype)
