@@ -19,7 +19,8 @@ at::Tensor tied_gate_recurrence(at::Tensor q, at::Tensor f_logit, at::Tensor v, 
                                 at::Tensor state, at::Tensor cu, at::Tensor start, at::Tensor slots);
 at::Tensor selective_scan(at::Tensor x, at::Tensor dt_raw, at::Tensor A_log, at::Tensor Bm, at::Tensor Cm,
                           at::Tensor D_skip, at::Tensor dt_bias, at::Tensor z, at::Tensor state, at::Tensor cu,
-                          at::Tensor start, at::Tensor slots, at::ScalarType out_dtype);
+                          at::Tensor start, at::Tensor slots, at::ScalarType out_dtype,
+                          c10::optional<at::Tensor> chunks, c10::optional<at::Tensor> seq_chunks);
 
 }  // namespace serving
 }  // namespace cai

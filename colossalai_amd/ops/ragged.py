@@ -32,6 +32,7 @@ class RaggedBatch:
     slots_host: List[int]
     page_size: int = 0
     _dense: Optional[tuple] = None  # memo of dense_context()
+    _scan_chunks: Optional[tuple] = None  # memo of the selective scan's chunk tables
 
     @property
     def num_seqs(self) -> int:

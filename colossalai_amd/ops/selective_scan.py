@@ -13,6 +13,13 @@ in its state slot (float32), is taken as zero for a sequence that starts at
 position 0, and is written back after the portion's last token, so a result
 does not depend on how a prompt was cut. The step size, both exponentials, the
 state and the read-out are float32.
+
+On the GPU a step with a long portion runs in chunks of ``CHUNK`` tokens that
+are scanned in parallel: once from a zero state for each chunk's end state and
+summed steps, a short sequential pass that carries the state from chunk to
+chunk (the recurrence is linear in the state and a chunk's decay is
+``exp(A * sum of its steps)``), and once more from each chunk's true incoming
+state for the output.
 """
 
 import torch
@@ -21,7 +28,22 @@ import torch.nn.functional as F
 from ._kernels import serving_state_kernels, use_serving_hip as use_hip
 from .ragged import RaggedBatch
 
-__all__ = ["selective_scan", "selective_scan_ref"]
+__all__ = ["selective_scan", "selective_scan_ref", "CHUNK", "CHUNKED_FROM"]
+
+CHUNK = 64           # tokens per chunk of the two-pass form (the kernel's own constant)
+CHUNKED_FROM = 256   # a step whose longest portion has at least this many tokens runs in chunks
+
+
+def _chunk_tables(batch: RaggedBatch):
+    """(chunks [K, 4] int32 = (sequence, first token, end token, 0), seq_chunks [B + 1]) on the device, one copy."""
+    rows, ranges = [], [0]
+    for b in range(batch.num_seqs):
+        lo, hi = batch.cu_host[b], batch.cu_host[b + 1]
+        for t in range(lo, hi, CHUNK):
+            rows += [b, t, min(t + CHUNK, hi), 0]
+        ranges.append(len(rows) // 4)
+    buf = torch.tensor(rows + ranges, dtype=torch.int32).to(batch.cu.device)
+    return buf[: len(rows)].view(-1, 4), buf[len(rows):]
 
 
 def selective_scan_ref(x, dt_raw, A_log, B, C, D_skip, dt_bias, z, state, batch: RaggedBatch, out_dtype=None):
@@ -45,6 +67,11 @@ def selective_scan(x, dt_raw, A_log, B, C, D_skip, dt_bias, z, state, batch: Rag
     (rows may be strided), A_log [C, S], D_skip and dt_bias [C] float32, state [slots, C, S] float32 (slot-strided
     allowed). Returns ``y * silu(z)`` [N, C] in ``out_dtype`` (default: z's)."""
     if use_hip(x):
+        chunks = seq_chunks = None
+        if batch.max_new >= CHUNKED_FROM:
+            if getattr(batch, "_scan_chunks", None) is None:
+                batch._scan_chunks = _chunk_tables(batch)     # once per step, shared by the step's layers
+            chunks, seq_chunks = batch._scan_chunks
         return serving_state_kernels().selective_scan(x, dt_raw, A_log, B, C, D_skip, dt_bias, z, state, batch.cu,
-                                                      batch.start, batch.slots, out_dtype or z.dtype)
+                                                      batch.start, batch.slots, out_dtype or z.dtype, chunks, seq_chunks)
     return selective_scan_ref(x, dt_raw, A_log, B, C, D_skip, dt_bias, z, state, batch, out_dtype)

@@ -143,11 +143,19 @@ def test_attention_block_summaries_and_talking_heads(dtype, H, G, D, Dv, window,
         torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dtype))
 
 
+def make_long_batch(device):
+    """A portion long enough for the chunked form (not a multiple of the chunk), beside a decode token, a short
+    continued portion and a second long, continued one."""
+    counts, starts, slots = [300, 1, 7, 257], [0, 63, 130, 40], [3, 0, 5, 1]
+    return (RaggedBatch.build(counts, starts, slots, device), RaggedBatch.build(counts, starts, slots, "cpu"), 0)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("C,S", [(320, 24), (64, 16), (100, 3), (48, 70), (8, 1)])
-def test_selective_scan(dtype, C, S):
+@pytest.mark.parametrize("long", [False, True])
+def test_selective_scan(dtype, C, S, long):
     torch.manual_seed(C + S)
-    dev, cpu, _ = make_batch("cuda")
+    dev, cpu, _ = make_long_batch("cuda") if long else make_batch("cuda")
     N = cpu.num_tokens
     x = torch.randn(N, C)
     packed = torch.randn(N, 2 * S + 5).to(dtype)
@@ -163,8 +171,9 @@ def test_selective_scan(dtype, C, S):
     pg, zg = packed.cuda(), z.cuda()
     got = scan_ops.selective_scan(x.cuda(), dt_raw.cuda(), A_log.cuda(), pg[:, 5 : 5 + S], pg[:, 5 + S :], D_skip.cuda(),
                                   dt_bias.cuda(), zg[:, C:], got_state, dev)
-    torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dtype))
-    torch.testing.assert_close(got_state.cpu(), want_state, rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **(tol(dtype) if not long or dtype == torch.bfloat16
+                                                                     else dict(rtol=2e-4, atol=2e-4)))
+    torch.testing.assert_close(got_state.cpu(), want_state, rtol=2e-4, atol=2e-4)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
