@@ -432,18 +432,31 @@ at::Tensor lerp_rows(at::Tensor a, at::Tensor b, double lam) {
 // o [N, H, G, Dv] float32 holds every query head's softmax weights applied to every key/value head's
 // values; mixing the weights of the heads is linear, so out[n, h, :] = sum_g talk[h, g] * o[n, g, kv(h), :]
 // with kv(h) = h / (H / G).
-template <typename TO>
+// One thread per (token, kv head c, run of RT heads of group c, channel): it reads the H cross outputs of its place
+// once and forms the rows of its RT heads (R = H / G heads in the group). RT = 8 reads the input once per eight heads
+// (large steps); RT = 1 gives a small step more threads.
+template <typename TO, int RT>
 __global__ __launch_bounds__(256) void talk_mix_kernel(TO* __restrict__ out, const float* __restrict__ o,
                                                        const float* __restrict__ talk, long N, int H, int G, int Dv) {
-  const long total = N * H * Dv;
+  const int R = H / G, runs = (R + RT - 1) / RT;
+  const long total = N * G * runs * Dv;
   for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
     const int d = (int)(i % Dv);
-    const int h = (int)(i / Dv % H);
-    const long n = i / Dv / H;
-    const int c = h / (H / G);
-    float acc = 0.0f;
-    for (int g = 0; g < H; ++g) acc += talk[h * H + g] * o[((n * H + g) * G + c) * Dv + d];
-    stf(out + i, acc);
+    const int r0 = (int)(i / Dv % runs) * RT;
+    const int c = (int)(i / Dv / runs % G);
+    const long n = i / Dv / runs / G;
+    float acc[RT];
+#pragma unroll
+    for (int r = 0; r < RT; ++r) acc[r] = 0.0f;
+    for (int g = 0; g < H; ++g) {
+      const float v = o[((n * H + g) * G + c) * Dv + d];
+#pragma unroll
+      for (int r = 0; r < RT; ++r)
+        if (r0 + r < R) acc[r] += talk[(c * R + r0 + r) * H + g] * v;
+    }
+#pragma unroll
+    for (int r = 0; r < RT; ++r)
+      if (r0 + r < R) stf(out + (n * H + c * R + r0 + r) * Dv + d, acc[r]);
   }
 }
 
@@ -456,9 +469,15 @@ at::Tensor talk_mix(at::Tensor o, at::Tensor talk, at::ScalarType out_dtype) {
   TORCH_CHECK(out_dtype == at::kFloat || out_dtype == at::kBFloat16);
   at::Tensor out = at::empty({N, H, Dv}, o.options().dtype(out_dtype));
   if (N == 0) return out;
+  const bool wide = N * H * Dv >= (1L << 20);
+  const long threads = wide ? N * G * ((H / G + 7) / 8) * Dv : N * H * Dv;
   SERVING_DISPATCH_ACT(out, TO, {
-    hipLaunchKernelGGL(talk_mix_kernel<TO>, dim3(capped_grid((N * H * Dv + 255) / 256, 8192)), dim3(256), 0, stream(),
-                       ptr<TO>(out), o.data_ptr<float>(), tk.data_ptr<float>(), N, H, G, Dv);
+    if (wide)
+      hipLaunchKernelGGL((talk_mix_kernel<TO, 8>), dim3(capped_grid((threads + 255) / 256, 8192)), dim3(256), 0, stream(),
+                         ptr<TO>(out), o.data_ptr<float>(), tk.data_ptr<float>(), N, H, G, Dv);
+    else
+      hipLaunchKernelGGL((talk_mix_kernel<TO, 1>), dim3(capped_grid((threads + 255) / 256, 8192)), dim3(256), 0, stream(),
+                         ptr<TO>(out), o.data_ptr<float>(), tk.data_ptr<float>(), N, H, G, Dv);
   });
   HIP_CHECK_LAST();
   return out;
