@@ -94,7 +94,7 @@ def latent_config(s: dict, experts: int = 32, top: int = 6) -> VitinexConfig:
 
 
 def pooled_config(s: dict, experts: int = 32, top: int = 6, window: int = 1024, pool: int = 64) -> TarulixConfig:
-    """Windowed attention (distance table of 32 rows, learned sink, values mixed with the first layer's) and the
+    """Windowed attention (distance table of 16 rows, learned sink, values mixed with the first layer's) and the
     parallel mixer (window + summaries of 64 positions + talking heads beside a selective scan of twice the width
     inside, 16 state places, 4 taps) in turn, Llama's head sizes; every layer carries routed gated experts of
     Mubutar's sizes (three matrices each, so two thirds of its hidden width) plus two identity experts."""
@@ -104,11 +104,11 @@ def pooled_config(s: dict, experts: int = 32, top: int = 6, window: int = 1024, 
     shared = (inter - top * ff + 127) // 128 * 128
     att = dict(bias_max=float(window), dim=D, heads=H, kv_heads=G, vdim=D, scale=1.0, mask=dict(size=window), v_mix=True)
     left = dict(dim=D, heads=H, kv_heads=G, vdim=D, scale=1.0, softcap=30.0, mask=dict(size=window, pool=pool),
-                rot=dict(base=250000.0, dims=D // 2))
+                rot=dict(base=10000.0, dims=D // 2))
     right = dict(conv=4, dt_rank=W // 16, inner=2 * W, state=16)
     mlp = dict(kind="moe", expert=dict(ff=ff), shared=dict(ff=shared), router=dict(experts=experts, identity=2, top=top))
     layers = [dict(type="attention", mixer=att, mlp=mlp) if i % 2 == 0 else
-              dict(type="parallel", mixer=dict(left=left, right=right, left_scale=0.8, right_scale=0.5), mlp=mlp)
+              dict(type="parallel", mixer=dict(left=left, right=right, left_scale=0.7, right_scale=0.6), mlp=mlp)
               for i in range(s["layers"])]
     return TarulixConfig(vocab=s["vocab"], width=W, layers=layers, norm_eps=1e-6)
 

@@ -284,11 +284,11 @@ class TarulixForCausalLM(nn.Module):
 
     def __init__(self, cfg: TarulixConfig, rel_rows: Optional[Dict[int, int]] = None):
         """``rel_rows`` maps a layer index to the rows of its distance table (a checkpoint's tensor shape gives it;
-        32 otherwise)."""
+        16 otherwise)."""
         super().__init__()
         self.config = cfg
         self.embed = nn.Embedding(cfg.vocab, cfg.width)
-        self.layers = nn.ModuleList([TarulixLayer(cfg, s, (rel_rows or {}).get(i, 32)) for i, s in enumerate(cfg.layers)])
+        self.layers = nn.ModuleList([TarulixLayer(cfg, s, (rel_rows or {}).get(i, 16)) for i, s in enumerate(cfg.layers)])
         self.final_norm = _scalar()
         self.head = nn.Linear(cfg.width, cfg.vocab, bias=False)
         first = None

@@ -22,7 +22,7 @@ class FalconPolicy(Policy):
         if self.shard_config.enable_tensor_parallelism and tp > 1:
             raise NotImplementedError(
                 "Falcon TP needs KV-head replication under multi-query attention; "
-                "use dp/zero/pp for Falcon this round"
+                "use dp/zero/pp for Falcon for now"
             )
         return {}
 

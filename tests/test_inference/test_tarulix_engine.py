@@ -195,7 +195,7 @@ def test_bfloat16_paths_agree_with_each_other_and_the_oracle():
     moe = dict(kind="moe", expert=dict(ff=32), router=dict(experts=6, identity=1, top=2), shared=dict(ff=32))
     cfg = dict(architecture="Tarulix", vocab=64, width=64, norm=dict(eps=1e-5),
                layers=[dict(type="attention", mixer=att, mlp=moe),
-                       dict(type="parallel", mixer=dict(left=left, right=right, left_scale=0.8, right_scale=0.5), mlp=moe),
+                       dict(type="parallel", mixer=dict(left=left, right=right, left_scale=0.9, right_scale=0.4), mlp=moe),
                        dict(type="attention", mixer=att, mlp=None)])
     W = {k: v.float() for k, v in O.random_checkpoint(cfg, seed=4).items()}
     toks = torch.randint(0, 64, (70,), generator=torch.Generator().manual_seed(9)).tolist()

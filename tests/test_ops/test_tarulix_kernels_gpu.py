@@ -43,16 +43,16 @@ def test_add_scaled_unit_norm(dtype, W, two):
     a = (torch.randn(N, W) * 2).to(dtype)
     b = (torch.randn(N, W) * 0.5).to(dtype) if two else None
     want_res = res.clone()
-    want = group_norm.add_scaled_unit_norm_ref(want_res, a, b, 0.8, 0.5, 1.7, 1e-6, dtype)
+    want = group_norm.add_scaled_unit_norm_ref(want_res, a, b, 0.9, 0.4, 1.7, 1e-6, dtype)
     got_res = res.cuda()
-    got = group_norm.add_scaled_unit_norm(got_res, a.cuda(), None if b is None else b.cuda(), 0.8, 0.5, 1.7, 1e-6, dtype)
+    got = group_norm.add_scaled_unit_norm(got_res, a.cuda(), None if b is None else b.cuda(), 0.9, 0.4, 1.7, 1e-6, dtype)
     torch.testing.assert_close(got_res.cpu(), want_res, rtol=2e-5, atol=2e-5)
     torch.testing.assert_close(got.cpu().float(), want.float(), **tol(dtype))
     assert group_norm.add_scaled_unit_norm(got_res, a.cuda(), None, 1.0, 0.0, 1.0, 1e-6, None) is None
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,D,dims", [(8, 64, 0), (4, 96, 24), (3, 40, 40), (2, 136, 64), (1, 320, 6)])
+@pytest.mark.parametrize("H,D,dims", [(8, 64, 0), (4, 80, 24), (3, 40, 40), (2, 136, 64), (1, 320, 6)])
 @pytest.mark.parametrize("eps", [1e-6, None])
 def test_rotate_halves_unit_norm(dtype, H, D, dims, eps):
     torch.manual_seed(D)
@@ -60,7 +60,7 @@ def test_rotate_halves_unit_norm(dtype, H, D, dims, eps):
     packed = (torch.randn(N, H * D + 24) * 2).to(dtype)   # heads side by side inside a wider row
     x = packed[:, 8 : 8 + H * D].view(N, H, D)
     pos = torch.randint(0, 5000, (N,), dtype=torch.int32)
-    freqs = pair_frequencies(250000.0, dims) if dims else None
+    freqs = pair_frequencies(40000.0, dims) if dims else None
     want = half_rotary.rotate_halves_unit_norm_ref(x, pos, freqs, eps)
     xg = packed.cuda()[:, 8 : 8 + H * D].view(N, H, D)
     got = half_rotary.rotate_halves_unit_norm(xg, pos.cuda(), None if freqs is None else freqs.cuda(), eps)
@@ -104,7 +104,7 @@ def test_paged_pool_write(dtype, P):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,G,D,Dv", [(8, 2, 64, 64), (4, 4, 40, 24), (6, 2, 96, 136), (2, 1, 20, 6)])
+@pytest.mark.parametrize("H,G,D,Dv", [(8, 2, 64, 32), (4, 4, 40, 24), (6, 2, 96, 136), (2, 1, 20, 6)])
 @pytest.mark.parametrize("window", [0, 7, 50])
 def test_attention_distance_table_and_learned_sink(dtype, H, G, D, Dv, window):
     torch.manual_seed(H * D + window)
@@ -122,7 +122,7 @@ def test_attention_distance_table_and_learned_sink(dtype, H, G, D, Dv, window):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,G,D,Dv", [(8, 4, 96, 96), (4, 1, 40, 24), (6, 6, 24, 136), (3, 3, 20, 6)])
+@pytest.mark.parametrize("H,G,D,Dv", [(8, 4, 96, 64), (4, 1, 40, 24), (6, 6, 24, 136), (3, 3, 20, 6)])
 @pytest.mark.parametrize("window,P", [(20, 16), (9, 4), (33, 6), (16, 40), (1, 1)])
 def test_attention_block_summaries_and_talking_heads(dtype, H, G, D, Dv, window, P):
     torch.manual_seed(H * D + window)
@@ -151,7 +151,7 @@ def make_long_batch(device):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("C,S", [(320, 24), (64, 16), (100, 3), (48, 70), (8, 1)])
+@pytest.mark.parametrize("C,S", [(192, 20), (64, 16), (100, 3), (48, 70), (8, 1)])
 @pytest.mark.parametrize("long", [False, True])
 def test_selective_scan(dtype, C, S, long):
     torch.manual_seed(C + S)
