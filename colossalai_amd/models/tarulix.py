@@ -152,7 +152,8 @@ class TarulixPooledAttention(_Attention):
     def __init__(self, width: int, c: dict, eps: float):
         super().__init__(width, c, eps)
         self.softcap = float(c.get("softcap") or 0.0)
-        self.summary_block = int(c["mask"]["pool"])
+        pool = c["mask"].get("pool")
+        self.summary_block = int(pool) if pool else None   # without a block length the window stands alone
         rot = c.get("rot") or {}
         self.rot_dims, self.rot_base = int(rot.get("dims", 0)), float(rot.get("base", 10000.0))
         if self.rot_dims % 2 or self.rot_dims > self.D:
@@ -168,9 +169,12 @@ class TarulixPooledAttention(_Attention):
         k = rotate_halves_unit_norm(p["k"].view(N, self.G, self.D), batch.positions, self.freqs, self.eps)
         kpool, vpool, ksum, vsum = pools
         paged_kv_write(k, p["v"].view(N, self.G, self.Dv), kpool, vpool, batch)
-        paged_pool_write(kpool, vpool, ksum, vsum, batch, self.summary_block)
+        pooled = None
+        if self.summary_block is not None:
+            paged_pool_write(kpool, vpool, ksum, vsum, batch, self.summary_block)
+            pooled = (ksum, vsum, self.summary_block)
         o = paged_attention(q, kpool, vpool, batch, self.scale, window=self.window, softcap=self.softcap,
-                            pooled=(ksum, vsum, self.summary_block), talk=self.talk)
+                            pooled=pooled, talk=self.talk)
         return self.o(o.reshape(N, self.H * self.Dv))
 
 
